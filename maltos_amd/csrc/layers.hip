@@ -1,0 +1,442 @@
+// HBM-bound layer kernels: RMSNorm, interleaved RoPE, SwiGLU.  Each is one coalesced pass with
+// 16-byte accesses; row statistics use 64-lane shuffle reductions.  Where the reference's eager ops
+// materialise an intermediate in bf16 the same rounding is reproduced here, so the forward results
+// are the reference's values and not merely close to them.
+#include "common.hpp"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / MLTS_WAVE;
+
+// ============================== RMSNorm ==================================================
+// One wavefront per row; a row is walked in chunks of 64 lanes x 16 bytes.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                               T* __restrict__ y, float* __restrict__ rstd_out,
+                                                               int64_t rows, int hidden, float eps) {
+  constexpr int N = Vec16<T>::N;
+  const int lane = threadIdx.x & (MLTS_WAVE - 1);
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + (threadIdx.x / MLTS_WAVE);
+  if (row >= rows) return;
+  const T* xr = x + row * hidden;
+  T* yr = y + row * hidden;
+  const int nvec = hidden / N;
+  float ss = 0.f;
+  for (int c = lane; c < nvec; c += MLTS_WAVE) {
+    Vec16<T> t = reinterpret_cast<const Vec16<T>*>(xr)[c];
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      float f = t.get(j);
+      ss += f * f;
+    }
+  }
+  ss = wave_sum(ss);
+  const float r = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  if (lane == 0 && rstd_out) rstd_out[row] = r;
+  for (int c = lane; c < nvec; c += MLTS_WAVE) {
+    Vec16<T> t = reinterpret_cast<const Vec16<T>*>(xr)[c];
+    Vec16<T> wv = reinterpret_cast<const Vec16<T>*>(w)[c];
+    Vec16<T> o;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      float n = round_to<T>(t.get(j) * r);  // (x * rsqrt(var + eps)).to(x.dtype)
+      o.set(j, wv.get(j) * n);              // weight * normed, rounded by set()
+    }
+    reinterpret_cast<Vec16<T>*>(yr)[c] = o;
+  }
+}
+
+// dx = r * (g - xhat * mean(g * xhat)), g = dy * w, xhat = x * r; per-block partial of
+// dw = sum_rows dy * xhat is written to dw_partial[block][hidden].
+// Each wave walks rows block*rows_per_block + wave, + kWaves, ...; lanes own fixed columns, so dw
+// partials live in registers (hidden <= 64 * N * kMaxChunks).
+constexpr int kMaxChunks = 8;
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                               const T* __restrict__ w, const float* __restrict__ rstd,
+                                                               T* __restrict__ dx, float* __restrict__ dw_partial,
+                                                               int64_t rows, int hidden, int rows_per_block) {
+  constexpr int N = Vec16<T>::N;
+  extern __shared__ float smem[];  // [kWaves][hidden]
+  const int lane = threadIdx.x & (MLTS_WAVE - 1);
+  const int wave = threadIdx.x / MLTS_WAVE;
+  const int nvec = hidden / N;
+  const int chunks = (nvec + MLTS_WAVE - 1) / MLTS_WAVE;
+  float dwacc[kMaxChunks][N];
+#pragma unroll
+  for (int c = 0; c < kMaxChunks; ++c)
+#pragma unroll
+    for (int j = 0; j < N; ++j) dwacc[c][j] = 0.f;
+
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rows_per_block;
+  int64_t row_end = row0 + rows_per_block;
+  if (row_end > rows) row_end = rows;
+  const float inv_h = 1.0f / static_cast<float>(hidden);
+  for (int64_t row = row0 + wave; row < row_end; row += kWaves) {
+    const float r = rstd[row];
+    const T* xr = x + row * hidden;
+    const T* dyr = dy + row * hidden;
+    T* dxr = dx + row * hidden;
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int col = lane + c * MLTS_WAVE;
+      if (c < chunks && col < nvec) {
+        Vec16<T> xv = reinterpret_cast<const Vec16<T>*>(xr)[col];
+        Vec16<T> dv = reinterpret_cast<const Vec16<T>*>(dyr)[col];
+        Vec16<T> wv = reinterpret_cast<const Vec16<T>*>(w)[col];
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          float xh = xv.get(j) * r;
+          float d = dv.get(j);
+          dwacc[c][j] += d * xh;
+          dot += d * wv.get(j) * xh;
+        }
+      }
+    }
+    dot = wave_sum(dot) * inv_h;
+#pragma unroll
+    for (int c = 0; c < kMaxChunks; ++c) {
+      const int col = lane + c * MLTS_WAVE;
+      if (c < chunks && col < nvec) {
+        Vec16<T> xv = reinterpret_cast<const Vec16<T>*>(xr)[col];
+        Vec16<T> dv = reinterpret_cast<const Vec16<T>*>(dyr)[col];
+        Vec16<T> wv = reinterpret_cast<const Vec16<T>*>(w)[col];
+        Vec16<T> o;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+          float xh = xv.get(j) * r;
+          o.set(j, r * (dv.get(j) * wv.get(j) - xh * dot));
+        }
+        reinterpret_cast<Vec16<T>*>(dxr)[col] = o;
+      }
+    }
+  }
+  // reduce the four waves' dw partials through LDS
+#pragma unroll
+  for (int c = 0; c < kMaxChunks; ++c) {
+    const int col = lane + c * MLTS_WAVE;
+    if (c < chunks && col < nvec) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) smem[wave * hidden + col * N + j] = dwacc[c][j];
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < hidden; i += kThreads) {
+    float s = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kWaves; ++wv) s += smem[wv * hidden + i];
+    dw_partial[static_cast<int64_t>(blockIdx.x) * hidden + i] = s;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void rmsnorm_dw_reduce_kernel(const float* __restrict__ dw_partial, int nblocks,
+                                                                     int hidden, T* __restrict__ dw) {
+  const int col = blockIdx.x * kThreads + threadIdx.x;
+  if (col >= hidden) return;
+  float s = 0.f;
+  for (int b = 0; b < nblocks; ++b) s += dw_partial[static_cast<int64_t>(b) * hidden + col];
+  dw[col] = from_f32<T>(s);
+}
+
+int rmsnorm_bwd_blocks(int64_t rows) {
+  int64_t b = (rows + 31) / 32;  // >= 32 rows per block keeps the partial buffer small
+  if (b > 1024) b = 1024;
+  if (b < 1) b = 1;
+  return static_cast<int>(b);
+}
+
+// ============================== RoPE =====================================================
+// One lane rotates the pairs inside one 16-byte vector of a [b, h, s, :] row.
+template <typename T, bool INVERSE>
+__global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
+                                                        T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
+                                                        const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
+                                                        int max_pos, const int32_t* __restrict__ positions,
+                                                        int position_offset, int B, int H, int S, int D) {
+  constexpr int N = Vec16<T>::N;
+  const int vec_per_row = D / N;
+  const int64_t total = static_cast<int64_t>(B) * S * H * vec_per_row;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx >= total) return;
+  // order (b, s, h, vec): neighbouring lanes touch neighbouring memory for [B, S, H, D] storage
+  const int vc = static_cast<int>(idx % vec_per_row);
+  int64_t rest = idx / vec_per_row;
+  const int h = static_cast<int>(rest % H);
+  rest /= H;
+  const int s = static_cast<int>(rest % S);
+  const int b = static_cast<int>(rest / S);
+  int pos = positions ? positions[static_cast<int64_t>(b) * S + s] : position_offset + s;
+  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);  // host validated; keeps reads in bounds
+  const T* xp = x + b * xsb + h * xsh + s * xss + vc * N;
+  T* yp = y + b * ysb + h * ysh + s * yss + vc * N;
+  Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(xp);
+  const T* cp = cos_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2);
+  const T* sp = sin_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2);
+  Vec16<T> o;
+#pragma unroll
+  for (int j = 0; j < N / 2; ++j) {
+    const float c = to_f32<T>(cp[j]);
+    float sn = to_f32<T>(sp[j]);
+    const float xe = xv.get(2 * j), xo = xv.get(2 * j + 1);
+    float oe, oo;
+    if (!INVERSE) {
+      oe = round_to<T>(xe * c) - round_to<T>(xo * sn);  // x_even * cos - x_odd * sin
+      oo = round_to<T>(xe * sn) + round_to<T>(xo * c);  // x_even * sin + x_odd * cos
+    } else {
+      oe = round_to<T>(xe * c) + round_to<T>(xo * sn);  // d_even * cos + d_odd * sin
+      oo = round_to<T>(xo * c) - round_to<T>(xe * sn);  // d_odd * cos - d_even * sin
+    }
+    o.set(2 * j, oe);
+    o.set(2 * j + 1, oo);
+  }
+  *reinterpret_cast<Vec16<T>*>(yp) = o;
+}
+
+// ============================== SwiGLU ===================================================
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float siluf_(float x) { return x / (1.0f + expf(-x)); }  // the form ATen evaluates
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                                              T* __restrict__ h, int64_t nvec) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < nvec; i += stride) {
+    Vec16<T> g = reinterpret_cast<const Vec16<T>*>(gate)[i];
+    Vec16<T> u = reinterpret_cast<const Vec16<T>*>(up)[i];
+    Vec16<T> o;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float gj = g.get(j);
+      const float act = round_to<T>(siluf_(gj));  // F.silu materialised in T
+      o.set(j, act * u.get(j));
+    }
+    reinterpret_cast<Vec16<T>*>(h)[i] = o;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const T* __restrict__ dh, const T* __restrict__ gate,
+                                                              const T* __restrict__ up, T* __restrict__ dgate,
+                                                              T* __restrict__ dup, int64_t nvec) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < nvec; i += stride) {
+    Vec16<T> d = reinterpret_cast<const Vec16<T>*>(dh)[i];
+    Vec16<T> g = reinterpret_cast<const Vec16<T>*>(gate)[i];
+    Vec16<T> u = reinterpret_cast<const Vec16<T>*>(up)[i];
+    Vec16<T> og, ou;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float gj = g.get(j), dj = d.get(j);
+      const float sg = sigmoidf_(gj);
+      ou.set(j, dj * (gj * sg));
+      og.set(j, dj * u.get(j) * (sg * (1.0f + gj * (1.0f - sg))));
+    }
+    reinterpret_cast<Vec16<T>*>(dgate)[i] = og;
+    reinterpret_cast<Vec16<T>*>(dup)[i] = ou;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_fwd_tail(const T* gate, const T* up, T* h, int64_t start, int64_t n) {
+  int64_t i = start + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const float gj = to_f32<T>(gate[i]);
+  const float act = round_to<T>(siluf_(gj));
+  h[i] = from_f32<T>(act * to_f32<T>(up[i]));
+}
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_tail(const T* dh, const T* gate, const T* up, T* dgate, T* dup,
+                                                            int64_t start, int64_t n) {
+  int64_t i = start + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i >= n) return;
+  const float gj = to_f32<T>(gate[i]), dj = to_f32<T>(dh[i]);
+  const float sg = sigmoidf_(gj);
+  dup[i] = from_f32<T>(dj * (gj * sg));
+  dgate[i] = from_f32<T>(dj * to_f32<T>(up[i]) * (sg * (1.0f + gj * (1.0f - sg))));
+}
+
+int stream_grid(int64_t nvec) {
+  int64_t b = (nvec + kThreads - 1) / kThreads;
+  if (b > 16384) b = 16384;
+  if (b < 1) b = 1;
+  return static_cast<int>(b);
+}
+
+template <typename T>
+int rmsnorm_fwd_t(const void* x, const void* w, void* y, float* rstd, int64_t rows, int hidden, float eps,
+                  hipStream_t st) {
+  const int64_t blocks = (rows + kWaves - 1) / kWaves;
+  hipLaunchKernelGGL(rmsnorm_fwd_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
+                     static_cast<const T*>(w), static_cast<T*>(y), rstd, rows, hidden, eps);
+  return mlts_check_launch("mlts_rmsnorm_fwd");
+}
+
+template <typename T>
+int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw, float* partial,
+                  int64_t rows, int hidden, hipStream_t st) {
+  const int blocks = rmsnorm_bwd_blocks(rows);
+  const int rows_per_block = static_cast<int>((rows + blocks - 1) / blocks);
+  const size_t smem = static_cast<size_t>(kWaves) * hidden * sizeof(float);
+  hipLaunchKernelGGL(rmsnorm_bwd_kernel<T>, dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy),
+                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,
+                     hidden, rows_per_block);
+  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
+                     partial, blocks, hidden, static_cast<T*>(dw));
+  return mlts_check_launch("mlts_rmsnorm_bwd");
+}
+
+template <typename T>
+int rope_t(const void* x, const int64_t* xs, void* y, const int64_t* ys, const void* ct, const void* sn, int max_pos,
+           const int32_t* positions, int off, int B, int H, int S, int D, int inverse, hipStream_t st) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t total = static_cast<int64_t>(B) * S * H * (D / N);
+  const int64_t blocks = (total + kThreads - 1) / kThreads;
+  if (blocks == 0) return MLTS_OK;
+  if (inverse)
+    hipLaunchKernelGGL((rope_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
+                       xs[0], xs[1], xs[2], static_cast<T*>(y), ys[0], ys[1], ys[2], static_cast<const T*>(ct),
+                       static_cast<const T*>(sn), max_pos, positions, off, B, H, S, D);
+  else
+    hipLaunchKernelGGL((rope_kernel<T, false>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
+                       xs[0], xs[1], xs[2], static_cast<T*>(y), ys[0], ys[1], ys[2], static_cast<const T*>(ct),
+                       static_cast<const T*>(sn), max_pos, positions, off, B, H, S, D);
+  return mlts_check_launch("mlts_rope");
+}
+
+template <typename T>
+int swiglu_fwd_t(const void* g, const void* u, void* h, int64_t n, bool vec, hipStream_t st) {
+  constexpr int N = Vec16<T>::N;
+  int64_t done = 0;
+  if (vec && n >= N) {
+    const int64_t nvec = n / N;
+    hipLaunchKernelGGL(swiglu_fwd_kernel<T>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const T*>(g),
+                       static_cast<const T*>(u), static_cast<T*>(h), nvec);
+    done = nvec * N;
+  }
+  if (done < n) {
+    const int64_t rem = n - done;
+    hipLaunchKernelGGL(swiglu_fwd_tail<T>, dim3((unsigned)((rem + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+                       static_cast<const T*>(g), static_cast<const T*>(u), static_cast<T*>(h), done, n);
+  }
+  return mlts_check_launch("mlts_swiglu_fwd");
+}
+
+template <typename T>
+int swiglu_bwd_t(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t n, bool vec,
+                 hipStream_t st) {
+  constexpr int N = Vec16<T>::N;
+  int64_t done = 0;
+  if (vec && n >= N) {
+    const int64_t nvec = n / N;
+    hipLaunchKernelGGL(swiglu_bwd_kernel<T>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const T*>(dh),
+                       static_cast<const T*>(g), static_cast<const T*>(u), static_cast<T*>(dg), static_cast<T*>(du),
+                       nvec);
+    done = nvec * N;
+  }
+  if (done < n) {
+    const int64_t rem = n - done;
+    hipLaunchKernelGGL(swiglu_bwd_tail<T>, dim3((unsigned)((rem + kThreads - 1) / kThreads)), dim3(kThreads), 0, st,
+                       static_cast<const T*>(dh), static_cast<const T*>(g), static_cast<const T*>(u),
+                       static_cast<T*>(dg), static_cast<T*>(du), done, n);
+  }
+  return mlts_check_launch("mlts_swiglu_bwd");
+}
+
+inline int elem_per_vec(int dtype) { return dtype == MLTS_BF16 ? 8 : 4; }
+inline bool known_dtype(int dtype) { return dtype == MLTS_BF16 || dtype == MLTS_F32; }
+
+}  // namespace
+
+extern "C" int mlts_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd_out, int64_t rows, int32_t hidden,
+                                float eps, int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "mlts_rmsnorm_fwd: unknown dtype %d", dtype);
+  MLTS_REQUIRE(rows >= 0 && hidden > 0, "mlts_rmsnorm_fwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
+  MLTS_REQUIRE(hidden % elem_per_vec(dtype) == 0, "mlts_rmsnorm_fwd: hidden=%d must be a multiple of %d", hidden,
+               elem_per_vec(dtype));
+  if (rows == 0) return MLTS_OK;
+  MLTS_REQUIRE(x && w && y, "mlts_rmsnorm_fwd: null pointer");
+  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(y), "mlts_rmsnorm_fwd: pointers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? rmsnorm_fwd_t<bf16_t>(x, w, y, rstd_out, rows, hidden, eps, st)
+                            : rmsnorm_fwd_t<float>(x, w, y, rstd_out, rows, hidden, eps, st);
+}
+
+extern "C" int64_t mlts_rmsnorm_bwd_workspace_bytes(int64_t rows, int32_t hidden) {
+  return static_cast<int64_t>(rmsnorm_bwd_blocks(rows)) * hidden * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int mlts_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw,
+                                void* workspace, int64_t workspace_bytes, int64_t rows, int32_t hidden, int32_t dtype,
+                                mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "mlts_rmsnorm_bwd: unknown dtype %d", dtype);
+  MLTS_REQUIRE(rows > 0 && hidden > 0, "mlts_rmsnorm_bwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
+  const int n = elem_per_vec(dtype);
+  MLTS_REQUIRE(hidden % n == 0, "mlts_rmsnorm_bwd: hidden=%d must be a multiple of %d", hidden, n);
+  MLTS_REQUIRE(hidden <= MLTS_WAVE * n * kMaxChunks, "mlts_rmsnorm_bwd: hidden=%d exceeds the supported maximum %d",
+               hidden, MLTS_WAVE * n * kMaxChunks);
+  MLTS_REQUIRE(dy && x && w && rstd && dx && dw && workspace, "mlts_rmsnorm_bwd: null pointer");
+  MLTS_REQUIRE(mlts_aligned16(dy) && mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(dx),
+               "mlts_rmsnorm_bwd: pointers must be 16-byte aligned");
+  MLTS_REQUIRE(workspace_bytes >= mlts_rmsnorm_bwd_workspace_bytes(rows, hidden),
+               "mlts_rmsnorm_bwd: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)mlts_rmsnorm_bwd_workspace_bytes(rows, hidden));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* partial = static_cast<float*>(workspace);
+  return dtype == MLTS_BF16 ? rmsnorm_bwd_t<bf16_t>(dy, x, w, rstd, dx, dw, partial, rows, hidden, st)
+                            : rmsnorm_bwd_t<float>(dy, x, w, rstd, dx, dw, partial, rows, hidden, st);
+}
+
+extern "C" int mlts_rope(const void* x, const int64_t x_stride[3], void* y, const int64_t y_stride[3],
+                         const void* cos_tab, const void* sin_tab, int32_t max_pos, const int32_t* positions,
+                         int32_t position_offset, int32_t B, int32_t H, int32_t S, int32_t D, int32_t dtype,
+                         int32_t inverse, mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "mlts_rope: unknown dtype %d", dtype);
+  MLTS_REQUIRE(B >= 0 && H >= 0 && S >= 0 && D > 0, "mlts_rope: bad shape");
+  const int n = elem_per_vec(dtype);
+  const int esz = dtype == MLTS_BF16 ? 2 : 4;
+  MLTS_REQUIRE(D % n == 0, "mlts_rope: head_dim=%d must be a multiple of %d", D, n);
+  if (B == 0 || H == 0 || S == 0) return MLTS_OK;
+  MLTS_REQUIRE(x && y && cos_tab && sin_tab && x_stride && y_stride, "mlts_rope: null pointer");
+  MLTS_REQUIRE(max_pos > 0, "mlts_rope: max_pos must be positive");
+  MLTS_REQUIRE(positions != nullptr || (position_offset >= 0 && position_offset + S <= max_pos),
+               "mlts_rope: positions [%d, %d) exceed the table (%d rows)", position_offset, position_offset + S, max_pos);
+  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(y), "mlts_rope: x and y must be 16-byte aligned");
+  for (int i = 0; i < 3; ++i)
+    MLTS_REQUIRE((x_stride[i] * esz) % 16 == 0 && (y_stride[i] * esz) % 16 == 0,
+                 "mlts_rope: strides must keep rows 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? rope_t<bf16_t>(x, x_stride, y, y_stride, cos_tab, sin_tab, max_pos, positions,
+                                             position_offset, B, H, S, D, inverse, st)
+                            : rope_t<float>(x, x_stride, y, y_stride, cos_tab, sin_tab, max_pos, positions,
+                                            position_offset, B, H, S, D, inverse, st);
+}
+
+extern "C" int mlts_swiglu_fwd(const void* gate, const void* up, void* h, int64_t n, int32_t dtype,
+                               mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "mlts_swiglu_fwd: unknown dtype %d", dtype);
+  MLTS_REQUIRE(n >= 0, "mlts_swiglu_fwd: n must be >= 0");
+  if (n == 0) return MLTS_OK;
+  MLTS_REQUIRE(gate && up && h, "mlts_swiglu_fwd: null pointer");
+  const bool vec = mlts_aligned16(gate) && mlts_aligned16(up) && mlts_aligned16(h);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? swiglu_fwd_t<bf16_t>(gate, up, h, n, vec, st) : swiglu_fwd_t<float>(gate, up, h, n, vec, st);
+}
+
+extern "C" int mlts_swiglu_bwd(const void* dh, const void* gate, const void* up, void* dgate, void* dup, int64_t n,
+                               int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "mlts_swiglu_bwd: unknown dtype %d", dtype);
+  MLTS_REQUIRE(n >= 0, "mlts_swiglu_bwd: n must be >= 0");
+  if (n == 0) return MLTS_OK;
+  MLTS_REQUIRE(dh && gate && up && dgate && dup, "mlts_swiglu_bwd: null pointer");
+  const bool vec = mlts_aligned16(dh) && mlts_aligned16(gate) && mlts_aligned16(up) && mlts_aligned16(dgate) &&
+                   mlts_aligned16(dup);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? swiglu_bwd_t<bf16_t>(dh, gate, up, dgate, dup, n, vec, st)
+                            : swiglu_bwd_t<float>(dh, gate, up, dgate, dup, n, vec, st);
+}
