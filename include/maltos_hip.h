@@ -97,7 +97,7 @@ int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_s
 
 /* Log-sum-exp merge of one block into the running fp32 state, rows [q_off, q_off + q_len):
  *   lse' = logaddexp(lse, lse_b); out' = out * exp(lse - lse') + out_b * exp(lse_b - lse'),
- * with exp(-inf - x) := 0 and rows where both are -inf left untouched.  Replaces
+ * with exp(-inf - x) := 0 (a row where both are -inf becomes 0 with lse -inf).  Replaces
  * _merge_attention_blocks / _exp_delta_or_zero (runtime/layers/functional.py:717-748).
  * out_acc fp32 [B, H, S, D] contiguous; lse_acc fp32 [B, H, S]; o_blk [B, H, q_len, D] of
  * blk_dtype with strides; lse_blk fp32 [B, H, q_len] contiguous. */

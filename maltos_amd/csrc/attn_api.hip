@@ -1,0 +1,245 @@
+// C-ABI entry points for attention: argument validation on the host, workspace carving, kernel
+// selection (bf16 head_dim 64/128 -> MFMA kernels, everything else -> generic fp32-ALU kernels) and
+// the log-sum-exp block merge.
+#include "attn_common.hpp"
+
+int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st);
+int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);
+int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32);
+int mlts_attn_generic_fwd(const AttnParams& p, int D, int dtype, int mode, hipStream_t st);
+int mlts_attn_generic_bwd(const AttnBwdParams& bp, int D, int dtype, int mode, hipStream_t st);
+int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const int64_t* os, float* delta, int B, int H,
+                    int S, int D, int dtype, hipStream_t st);
+
+namespace {
+
+inline int64_t align256(int64_t x) { return (x + 255) & ~255LL; }
+inline int esize(int dtype) { return dtype == MLTS_BF16 ? 2 : 4; }
+
+bool uses_mfma(const mlts_attn_shape* s) { return s->dtype == MLTS_BF16 && (s->D == 64 || s->D == 128); }
+
+bool strides_aligned(const int64_t* st, int es) {
+  for (int i = 0; i < 3; ++i)
+    if ((st[i] * es) % 16 != 0) return false;
+  return true;
+}
+
+const char* shape_problem(const mlts_attn_shape* s) {
+  if (!s) return "shape is null";
+  if (s->dtype != MLTS_BF16 && s->dtype != MLTS_F32) return "dtype must be MLTS_F32 or MLTS_BF16";
+  if (s->B < 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Sq < 0 || s->Sk < 0 || s->D <= 0) return "negative or zero dimension";
+  if (s->Hq % s->Hkv != 0) return "Hq must be a multiple of Hkv";
+  if (s->D > 256) return "head_dim > 256 is not supported";
+  if (s->mask_mode < MLTS_MASK_NONE || s->mask_mode > MLTS_MASK_DOC) return "unknown mask_mode";
+  if (!(s->scale > 0.f)) return "softmax scale must be positive";
+  if (s->mask_mode == MLTS_MASK_DOC && !(s->q_pos && s->k_pos && s->q_seq && s->k_seq))
+    return "MLTS_MASK_DOC needs q_pos, k_pos, q_seq and k_seq";
+  if (uses_mfma(s)) {
+    if (!strides_aligned(s->q_stride, 2) || !strides_aligned(s->k_stride, 2) || !strides_aligned(s->v_stride, 2) ||
+        !strides_aligned(s->o_stride, 2))
+      return "bf16 MFMA path needs strides that keep rows 16-byte aligned";
+  }
+  return nullptr;
+}
+
+int64_t stats_bytes(const mlts_attn_shape* s) {
+  if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return 0;
+  const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
+  return align256(s->B * nq * 16) + align256(s->B * nk * 16);
+}
+
+void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o,
+                 float* lse) {
+  p.q = q;
+  p.k = k;
+  p.v = v;
+  p.o = o;
+  p.lse = lse;
+  for (int i = 0; i < 3; ++i) {
+    p.qs[i] = s->q_stride[i];
+    p.ks[i] = s->k_stride[i];
+    p.vs[i] = s->v_stride[i];
+    p.os[i] = s->o_stride[i];
+  }
+  p.B = s->B;
+  p.Hq = s->Hq;
+  p.Hkv = s->Hkv;
+  p.Sq = s->Sq;
+  p.Sk = s->Sk;
+  p.scale = s->scale;
+  p.scale_log2 = s->scale * kLog2e;
+  p.causal_off = s->Sk - s->Sq;
+  p.q_pos = s->q_pos;
+  p.k_pos = s->k_pos;
+  p.q_seq = s->q_seq;
+  p.k_seq = s->k_seq;
+  p.q_stats = nullptr;
+  p.k_stats = nullptr;
+  p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
+  p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
+  p.nqt = 0;
+}
+
+// Carves the tile statistics out of the front of the workspace and launches their kernels.
+char* setup_stats(AttnParams& p, const mlts_attn_shape* s, char* ws, hipStream_t st) {
+  if (stats_bytes(s) == 0) return ws;
+  int4* qst = reinterpret_cast<int4*>(ws);
+  ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * 16);
+  int4* kst = reinterpret_cast<int4*>(ws);
+  ws += align256(static_cast<int64_t>(s->B) * p.nk_stats * 16);
+  mlts_launch_tile_stats(s->q_pos, s->q_seq, s->B, s->Sq, qst, st);
+  mlts_launch_tile_stats(s->k_pos, s->k_seq, s->B, s->Sk, kst, st);
+  p.q_stats = qst;
+  p.k_stats = kst;
+  return ws;
+}
+
+// A row (D/4 vectors) is owned by G = 2^k <= 64 adjacent lanes of ONE wavefront, so the row's
+// lse_acc is read by all of them before one of them rewrites it (program order inside a wave).
+template <typename T>
+__global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc, float* __restrict__ lse_acc,
+                                                    const T* __restrict__ o_blk, int64_t bs0, int64_t bs1, int64_t bs2,
+                                                    const float* __restrict__ lse_blk, int H, int S, int D, int q_off,
+                                                    int q_len, int64_t total_rows, int G) {
+  const int vec_per_row = D >> 2;
+  const int rows_per_block = 256 / G;
+  const int64_t rowi = static_cast<int64_t>(blockIdx.x) * rows_per_block + threadIdx.x / G;
+  const int sub = threadIdx.x % G;
+  if (rowi >= total_rows) return;
+  const int i = static_cast<int>(rowi % q_len);
+  const int64_t bh = rowi / q_len;
+  const int h = static_cast<int>(bh % H), b = static_cast<int>(bh / H);
+  const int64_t arow = bh * S + q_off + i;
+  const float la = lse_acc[arow], lb = lse_blk[bh * q_len + i];
+  const float mx = fmaxf(la, lb);
+  float ln = -INFINITY, pa = 0.f, pb = 0.f;
+  if (mx != -INFINITY) {
+    ln = mx + log1pf(expf(-fabsf(la - lb)));  // logaddexp; -inf on one side returns the other side
+    pa = isfinite(la) ? expf(la - ln) : 0.f;
+    pb = isfinite(lb) ? expf(lb - ln) : 0.f;
+  }
+  const T* bp = o_blk + b * bs0 + h * bs1 + static_cast<int64_t>(i) * bs2;
+  for (int vc = sub; vc < vec_per_row; vc += G) {
+    const f32x4 acc = reinterpret_cast<const f32x4*>(out_acc + arow * D)[vc];
+    f32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = acc[e] * pa + to_f32<T>(bp[vc * 4 + e]) * pb;
+    reinterpret_cast<f32x4*>(out_acc + arow * D)[vc] = r;
+  }
+  if (sub == 0) lse_acc[arow] = ln;
+}
+
+}  // namespace
+
+extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return shape_problem(s); }
+
+extern "C" int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s) {
+  if (shape_problem(s)) return -1;
+  return stats_bytes(s);
+}
+
+extern "C" int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32) {
+  if (shape_problem(s)) return -1;
+  const int64_t delta = align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
+  int64_t extra = 0;
+  if (uses_mfma(s)) extra = mlts_attn_bwd_bf16_workspace(s, accumulate_f32);
+  return stats_bytes(s) + delta + extra;
+}
+
+extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o, float* lse,
+                             void* workspace, int64_t workspace_bytes, mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_fwd: %s", why);
+  if (s->B == 0 || s->Sq == 0) return MLTS_OK;
+  MLTS_REQUIRE(q && o && lse, "mlts_attn_fwd: q, o, lse must be non-null");
+  MLTS_REQUIRE(s->Sk == 0 || (k && v), "mlts_attn_fwd: k, v must be non-null");
+  const int64_t need = stats_bytes(s);
+  MLTS_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), "mlts_attn_fwd: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  AttnParams p;
+  fill_params(p, s, q, k, v, o, lse);
+  if (uses_mfma(s)) {
+    MLTS_REQUIRE(mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) && mlts_aligned16(o),
+                 "mlts_attn_fwd: q, k, v, o must be 16-byte aligned");
+    setup_stats(p, s, static_cast<char*>(workspace), st);
+    return mlts_attn_fwd_bf16(p, s->D, s->mask_mode, st);
+  }
+  return mlts_attn_generic_fwd(p, s->D, s->dtype, s->mask_mode, st);
+}
+
+extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
+                             const void* k, const void* v, const void* o, const float* lse, void* dq,
+                             const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,
+                             const int64_t dv_stride[3], int accumulate_f32, void* workspace, int64_t workspace_bytes,
+                             mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_bwd: %s", why);
+  if (s->B == 0 || (s->Sq == 0 && s->Sk == 0)) return MLTS_OK;
+  MLTS_REQUIRE(dout && q && k && v && o && lse && dq && dk && dv, "mlts_attn_bwd: null tensor pointer");
+  MLTS_REQUIRE(do_stride && dq_stride && dk_stride && dv_stride, "mlts_attn_bwd: null stride pointer");
+  const int64_t need = mlts_attn_bwd_workspace_bytes(s, accumulate_f32);
+  MLTS_REQUIRE(workspace && workspace_bytes >= need, "mlts_attn_bwd: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  AttnBwdParams bp;
+  fill_params(bp.a, s, q, k, v, const_cast<void*>(o), const_cast<float*>(lse));
+  char* ws = setup_stats(bp.a, s, static_cast<char*>(workspace), st);
+  float* delta = reinterpret_cast<float*>(ws);
+  ws += align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
+  bp.dout = dout;
+  bp.delta = delta;
+  bp.dq_acc = static_cast<float*>(dq);
+  bp.dk = dk;
+  bp.dv = dv;
+  for (int i = 0; i < 3; ++i) {
+    bp.dos[i] = do_stride[i];
+    bp.dqs[i] = dq_stride[i];
+    bp.dks[i] = dk_stride[i];
+    bp.dvs[i] = dv_stride[i];
+  }
+  bp.accumulate_f32 = accumulate_f32 ? 1 : 0;
+  bp.nkt = 0;
+  if (s->Sq > 0) {
+    int rc = mlts_attn_delta(dout, do_stride, o, s->o_stride, delta, s->B, s->Hq, s->Sq, s->D, s->dtype, st);
+    if (rc != MLTS_OK) return rc;
+  }
+  if (uses_mfma(s)) {
+    MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
+                     mlts_aligned16(dq) && mlts_aligned16(dk) && mlts_aligned16(dv),
+                 "mlts_attn_bwd: tensors must be 16-byte aligned");
+    const int es_out = accumulate_f32 ? 4 : 2;
+    MLTS_REQUIRE(strides_aligned(do_stride, 2) && strides_aligned(dq_stride, es_out) &&
+                     strides_aligned(dk_stride, es_out) && strides_aligned(dv_stride, es_out),
+                 "mlts_attn_bwd: strides must keep rows 16-byte aligned");
+    return mlts_attn_bwd_bf16(bp, s->D, s->mask_mode, ws, st);
+  }
+  return mlts_attn_generic_bwd(bp, s->D, s->dtype, s->mask_mode, st);
+}
+
+extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk, const int64_t o_blk_stride[3],
+                               int32_t blk_dtype, const float* lse_blk, int32_t B, int32_t H, int32_t S, int32_t D,
+                               int32_t q_off, int32_t q_len, mlts_stream_t stream) {
+  MLTS_REQUIRE(blk_dtype == MLTS_BF16 || blk_dtype == MLTS_F32, "mlts_attn_merge: unknown dtype %d", blk_dtype);
+  MLTS_REQUIRE(B >= 0 && H >= 0 && S >= 0 && D > 0 && q_off >= 0 && q_len >= 0 && q_off + q_len <= S,
+               "mlts_attn_merge: rows [%d, %d) do not fit S=%d", q_off, q_off + q_len, S);
+  MLTS_REQUIRE(D % 4 == 0, "mlts_attn_merge: head_dim must be a multiple of 4");
+  if (B == 0 || H == 0 || q_len == 0) return MLTS_OK;
+  MLTS_REQUIRE(out_acc && lse_acc && o_blk && lse_blk && o_blk_stride, "mlts_attn_merge: null pointer");
+  MLTS_REQUIRE(mlts_aligned16(out_acc), "mlts_attn_merge: out_acc must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total_rows = static_cast<int64_t>(B) * H * q_len;
+  int G = 1;
+  while (G < D / 4 && G < 64) G <<= 1;
+  const int rows_per_block = 256 / G;
+  const int64_t blocks = (total_rows + rows_per_block - 1) / rows_per_block;
+  if (blk_dtype == MLTS_BF16)
+    hipLaunchKernelGGL(merge_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, out_acc, lse_acc,
+                       static_cast<const bf16_t*>(o_blk), o_blk_stride[0], o_blk_stride[1], o_blk_stride[2], lse_blk, H, S,
+                       D, q_off, q_len, total_rows, G);
+  else
+    hipLaunchKernelGGL(merge_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, out_acc, lse_acc,
+                       static_cast<const float*>(o_blk), o_blk_stride[0], o_blk_stride[1], o_blk_stride[2], lse_blk, H, S,
+                       D, q_off, q_len, total_rows, G);
+  return mlts_check_launch("mlts_attn_merge");
+}

@@ -1,0 +1,59 @@
+// Shared pieces of the attention kernels: kernel parameter block, mask predicate, per-tile
+// position/sequence statistics used to skip or fast-path whole 64-key tiles.
+#pragma once
+#include "common.hpp"
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+constexpr int kAttnTile = 64;  // granularity of the tile statistics (queries per wave, keys per tile)
+
+struct AttnParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;
+  int64_t qs[3], ks[3], vs[3], os[3];
+  int B, Hq, Hkv, Sq, Sk;
+  float scale;        // softmax scale
+  float scale_log2;   // scale * log2(e)
+  int causal_off;     // Sk - Sq: key j visible to query i iff j <= i + causal_off
+  const int32_t* q_pos;
+  const int32_t* k_pos;
+  const int32_t* q_seq;
+  const int32_t* k_seq;
+  const int4* q_stats;  // [B, ceil(Sq/64)] (min_pos, max_pos, min_seq, max_seq)
+  const int4* k_stats;  // [B, ceil(Sk/64)]
+  int nq_stats, nk_stats;
+  int nqt;              // query tiles per (batch, head) for the launched kernel
+};
+
+// Backward-only extras.
+struct AttnBwdParams {
+  AttnParams a;
+  const void* dout;
+  int64_t dos[3];
+  const float* delta;  // [B, Hq, Sq] rowsum(dO * O)
+  float* dq_acc;       // fp32 [B, Hq, Sq, D] accumulated with atomics (contiguous or caller strides)
+  int64_t dqs[3];
+  void* dk;
+  void* dv;
+  int64_t dks[3], dvs[3];
+  int accumulate_f32;  // dk/dv are fp32 and added to
+  int nkt;             // key tiles per (batch, kv head)
+};
+
+enum TileClass { TILE_SKIP = 0, TILE_FULL = 1, TILE_MASKED = 2 };
+
+// Classification of a (64-query group, 64-key tile) pair from the statistics, MLTS_MASK_DOC.
+__device__ __forceinline__ int classify_doc_tile(const int4 qs, const int4 ks) {
+  // nothing visible: every key is later than every query, or the sequence-id ranges are disjoint,
+  // or every query is padding
+  if (ks.x > qs.y || ks.w < qs.z || ks.z > qs.w || qs.w < 0) return TILE_SKIP;
+  // everything visible: all keys precede all queries and a single non-padding sequence id
+  if (ks.y <= qs.x && qs.z == qs.w && ks.z == ks.w && ks.z == qs.z && qs.z >= 0) return TILE_FULL;
+  return TILE_MASKED;
+}
+
+void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);

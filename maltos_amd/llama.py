@@ -1,0 +1,208 @@
+"""LLaMA decoder path on the HIP kernels.
+
+Counterpart of the reference's models/llama.py:30-330 with identical module and parameter names
+(embed_tokens, layers.N.self_attn.{q,k,v,o}_proj, layers.N.mlp.{gate,up,down}_proj,
+layers.N.{input,post_attention}_layernorm, norm, lm_head), so state dicts are interchangeable.
+RMSNorm, RoPE, attention, SwiGLU and the loss are the `maltos::` custom ops; the projections and the
+embedding stay on the vendor GEMM library through torch.  Attention consumes the [B, H, S, D] views
+of the projection outputs in place and keeps K/V at their native head count.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .attention_backend import AttentionBackend, causal_attention, validate_attention_backend
+from .attn_masking_utils import canonical_position_ids, canonical_sequence_ids
+from .constants import (HIDDEN_STATES_KEY, INPUT_IDS_KEY, LABELS_KEY, LOSS_WEIGHT_KEY, POSITION_IDS_KEY,
+                        POSITION_OFFSET_KEY, SEQUENCE_IDS_KEY)
+from .losses import causal_cross_entropy
+
+
+@dataclass(frozen=True)
+class LlamaConfig:
+    vocab_size: int
+    hidden_size: int = 512
+    intermediate_size: int = 2048
+    num_hidden_layers: int = 8
+    num_attention_heads: int = 8
+    num_key_value_heads: int | None = None
+    max_position_embeddings: int = 2048
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 10000.0
+    tie_word_embeddings: bool = False
+    attention_backend: str = AttentionBackend.HIP
+
+    def __post_init__(self) -> None:
+        validate_attention_backend(self.attention_backend)
+
+
+class LlamaRMSNorm(nn.Module):
+    def __init__(self, hidden_size: int, eps: float) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rms_norm(x, self.weight, self.eps)
+
+
+class LlamaRotaryEmbedding(nn.Module):
+    """cos/sin tables [max_position_embeddings, head_dim / 2], built in fp32 and cast with the module."""
+
+    def __init__(self, head_dim: int, max_position_embeddings: int, base: float) -> None:
+        super().__init__()
+        exponents = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
+        angles = torch.arange(max_position_embeddings, dtype=torch.float32)[:, None] * (base ** -exponents)[None, :]
+        self.register_buffer("cos", torch.cos(angles), persistent=False)
+        self.register_buffer("sin", torch.sin(angles), persistent=False)
+
+    def tables(self, dtype: torch.dtype, device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
+        if self.cos.dtype != dtype or self.cos.device != device:
+            # fp32 -> dtype is the single rounding the reference applies (cos.to(x.dtype))
+            return self.cos.to(device=device, dtype=dtype), self.sin.to(device=device, dtype=dtype)
+        return self.cos, self.sin
+
+
+class HipAttentionCore(nn.Module):
+    """`attn_core` of LlamaAttention: (q, k, v, position_offset, position_ids, sequence_ids) -> out."""
+
+    preserves_native_gqa = True
+
+    def __init__(self, attention_backend: str = AttentionBackend.HIP) -> None:
+        super().__init__()
+        self.attention_backend = validate_attention_backend(attention_backend)
+
+    def forward(self, q, k, v, position_offset: int, position_ids=None, sequence_ids=None) -> torch.Tensor:
+        positions = sequences = None
+        if position_ids is not None or sequence_ids is not None:
+            positions = canonical_position_ids(position_ids, batch_size=q.size(0), seq_len=q.size(-2),
+                                               position_offset=position_offset, device=q.device)
+            sequences = canonical_sequence_ids(sequence_ids, batch_size=q.size(0), seq_len=q.size(-2), device=q.device)
+        return causal_attention(q, k, v, attention_backend=self.attention_backend, warning_prefix="LlamaAttention",
+                                q_positions=positions, k_positions=positions, q_sequence_ids=sequences,
+                                k_sequence_ids=sequences, flash_varlen_mode="same_length")
+
+
+class LlamaAttention(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        if config.hidden_size % config.num_attention_heads != 0:
+            raise ValueError("hidden_size must be divisible by num_attention_heads")
+        self.num_heads = config.num_attention_heads
+        self.num_kv_heads = config.num_key_value_heads or config.num_attention_heads
+        if self.num_heads % self.num_kv_heads != 0:
+            raise ValueError("num_attention_heads must be divisible by num_key_value_heads")
+        self.head_dim = config.hidden_size // config.num_attention_heads
+        self.rotary_emb = LlamaRotaryEmbedding(self.head_dim, config.max_position_embeddings, config.rope_theta)
+        self.q_proj = nn.Linear(config.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.o_proj = nn.Linear(config.hidden_size, config.hidden_size, bias=False)
+        self.attn_core = HipAttentionCore(config.attention_backend)
+
+    def forward(self, x: torch.Tensor, *, position_offset: int = 0, position_ids: torch.Tensor | None = None,
+                sequence_ids: torch.Tensor | None = None) -> torch.Tensor:
+        batch, seq_len, _ = x.shape
+        cos, sin = self.rotary_emb.tables(x.dtype, x.device)
+        rope_pos = None
+        if position_ids is not None:
+            rope_pos = canonical_position_ids(position_ids, batch_size=batch, seq_len=seq_len, position_offset=0,
+                                              device=x.device)
+        # [B, S, H*D] -> [B, H, S, D] views; no copies until the kernels read them
+        q = self.q_proj(x).view(batch, seq_len, self.num_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
+        q = ops.rope(q, cos, sin, positions=rope_pos, position_offset=position_offset)
+        k = ops.rope(k, cos, sin, positions=rope_pos, position_offset=position_offset)
+        if not getattr(self.attn_core, "preserves_native_gqa", False) and self.num_heads != self.num_kv_heads:
+            rep = self.num_heads // self.num_kv_heads
+            k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+        vo = self.attn_core(q, k, v, position_offset, position_ids, sequence_ids)
+        return self.o_proj(vo.transpose(1, 2).reshape(batch, seq_len, self.num_heads * self.head_dim))
+
+
+class LlamaMLP(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(ops.swiglu(self.gate_proj(x), self.up_proj(x)))
+
+
+class LlamaDecoderLayer(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        self.self_attn = LlamaAttention(config)
+        self.mlp = LlamaMLP(config)
+        self.input_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, x: torch.Tensor, position_offset: int = 0, position_ids: torch.Tensor | None = None,
+                sequence_ids: torch.Tensor | None = None) -> torch.Tensor:
+        x = x + self.self_attn(self.input_layernorm(x), position_offset=position_offset, position_ids=position_ids,
+                               sequence_ids=sequence_ids)
+        return x + self.mlp(self.post_attention_layernorm(x))
+
+
+class LlamaForCausalLM(nn.Module):
+    def __init__(self, config: LlamaConfig) -> None:
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList([LlamaDecoderLayer(config) for _ in range(config.num_hidden_layers)])
+        self.norm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.embed_tokens.weight
+
+    def forward(self, batch):
+        """Accepts the reference's batch forms: dict with the constants' keys, (input_ids, labels), or input_ids.
+        Returns the scalar loss when labels are given (already aligned, no shift), else the logits."""
+        hidden_states = position_ids = sequence_ids = loss_weight = labels = None
+        position_offset = 0
+        if isinstance(batch, dict):
+            input_ids = batch.get(INPUT_IDS_KEY)
+            hidden_states = batch.get(HIDDEN_STATES_KEY)
+            labels = batch.get(LABELS_KEY)
+            position_offset = int(batch.get(POSITION_OFFSET_KEY, 0))
+            position_ids = batch.get(POSITION_IDS_KEY)
+            sequence_ids = batch.get(SEQUENCE_IDS_KEY)
+            loss_weight = batch.get(LOSS_WEIGHT_KEY)
+        elif isinstance(batch, (tuple, list)):
+            input_ids, labels = batch
+        else:
+            input_ids = batch
+        if hidden_states is not None:
+            x = hidden_states
+        elif input_ids is None:
+            raise ValueError("LlamaForCausalLM requires input_ids or hidden_states")
+        else:
+            x = self.embed_tokens(input_ids)
+        for layer in self.layers:
+            x = layer(x, position_offset=position_offset, position_ids=position_ids, sequence_ids=sequence_ids)
+        logits = self.lm_head(self.norm(x))
+        if labels is None:
+            return logits
+        if input_ids is not None and labels.shape != input_ids.shape:
+            raise ValueError(f"labels shape must match input_ids shape, got {labels.shape} vs {input_ids.shape}")
+        loss = causal_cross_entropy(logits, labels)
+        return loss if loss_weight is None else loss * float(loss_weight)
+
+    def context_parallel_spec(self) -> list[str]:
+        """Module paths whose `attn_core` a context-parallel plugin swaps (reference :311-314)."""
+        return [f"layers.{i}.self_attn" for i in range(len(self.layers))]
+
+    def flops_per_token(self) -> float:
+        """The reference's estimator (:319-330): 3 x forward, attention counted non-causal."""
+        c = self.config
+        h, i, s, v = c.hidden_size, c.intermediate_size, c.max_position_embeddings, c.vocab_size
+        per_layer = 6 * h * h + 2 * h * h + 6 * h * i + 4 * s * h
+        return float(3 * (c.num_hidden_layers * per_layer + 2 * h * v))

@@ -1,0 +1,139 @@
+"""Zigzag ring (context-parallel) block attention: one rank's compute on one GPU.
+
+Counterpart of the reference's flash ring path (runtime/layers/functional.py:619-645,751-820,
+1012-1166 and RingAttentionCore, runtime/layers/ring_attention.py:21-113).  A rank holds the local
+Q/K/V chunk in zigzag layout and, ring step by ring step, the K/V chunk of rank (rank - step) mod W:
+    step 0        square causal block on the local chunk
+    step <= rank  all local queries x the FRONT half of the remote chunk, no mask
+    step >  rank  the TAIL half of the local queries x the whole remote chunk, no mask
+Block outputs are merged in fp32 with a log-sum-exp merge; the backward pass re-runs the same
+schedule with the GLOBAL out / LSE and accumulates dQ and the per-chunk dK/dV in fp32.
+
+What moves K/V between ranks is a separate concern (the reference uses P2P send/recv): here it is
+the `kv_source` callable, which returns the chunk a step needs.  On one GPU the chunks are simply
+resident; nothing in this module touches torch.distributed.
+"""
+from __future__ import annotations
+
+from typing import Callable, Sequence
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .attention_backend import AttentionBackend, causal_attention, validate_attention_backend
+from .attn_masking_utils import canonical_position_ids, canonical_sequence_ids
+from .flash_utils import flash_attn_dense_with_lse
+
+KvChunk = tuple[torch.Tensor, torch.Tensor]
+
+
+def zigzag_ring_schedule(rank: int, world_size: int) -> list[tuple[int, str]]:
+    """[(source rank of the K/V chunk, block kind)] for ring steps 0..W-1."""
+    if not 0 <= rank < world_size:
+        raise ValueError(f"rank {rank} outside world of {world_size}")
+    plan = []
+    for step in range(world_size):
+        kind = "causal" if step == 0 else ("front_kv" if step <= rank else "tail_q")
+        plan.append(((rank - step) % world_size, kind))
+    return plan
+
+
+class _ZigzagRingFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q: torch.Tensor, rank: int, world_size: int, *kv_flat: torch.Tensor):
+        if len(kv_flat) != 2 * world_size:
+            raise ValueError(f"expected {2 * world_size} K/V tensors, got {len(kv_flat)}")
+        seq = q.size(-2)
+        if seq % 2:
+            raise ValueError(f"zigzag ring attention requires an even local sequence length, got {seq}")
+        half = seq // 2
+        running_out = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+        for src, kind in zigzag_ring_schedule(rank, world_size):
+            k, v = kv_flat[2 * src], kv_flat[2 * src + 1]
+            if kind == "causal":
+                blk = flash_attn_dense_with_lse(q, k, v, causal=True)
+                ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, 0)
+            elif kind == "front_kv":
+                blk = flash_attn_dense_with_lse(q, k[:, :, :half], v[:, :, :half], causal=False)
+                ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, 0)
+            else:
+                blk = flash_attn_dense_with_lse(q[:, :, half:], k, v, causal=False)
+                ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, half)
+        out = running_out.to(dtype=kv_flat[1].dtype)
+        ctx.save_for_backward(q, out, running_lse, *kv_flat)
+        ctx.rank, ctx.world_size = rank, world_size
+        ctx.mark_non_differentiable(running_lse)
+        return out, running_lse
+
+    @staticmethod
+    def backward(ctx, dout: torch.Tensor, _dlse):
+        q, out, lse, *kv_flat = ctx.saved_tensors
+        rank, world_size = ctx.rank, ctx.world_size
+        half = q.size(-2) // 2
+        dout = dout.contiguous()
+        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        grads: list[torch.Tensor | None] = [None] * (2 * world_size)
+        for src, kind in zigzag_ring_schedule(rank, world_size):
+            k, v = kv_flat[2 * src], kv_flat[2 * src + 1]
+            dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
+            dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+            if kind == "causal":
+                ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dk, dv, mask_mode=ops.MASK_CAUSAL)
+            elif kind == "front_kv":
+                ops.attention_backward_accumulate(dout, q, k[:, :, :half], v[:, :, :half], out, lse, dq, dk[:, :, :half],
+                                                  dv[:, :, :half], mask_mode=ops.MASK_NONE)
+            else:
+                ops.attention_backward_accumulate(dout[:, :, half:], q[:, :, half:], k, v, out[:, :, half:],
+                                                  lse[:, :, half:].contiguous(), dq[:, :, half:], dk, dv,
+                                                  mask_mode=ops.MASK_NONE)
+            grads[2 * src] = dk.to(k.dtype)
+            grads[2 * src + 1] = dv.to(v.dtype)
+        return (dq.to(q.dtype), None, None, *grads)
+
+
+def zigzag_ring_attention(q: torch.Tensor, kv_chunks: Sequence[KvChunk], *, rank: int, world_size: int,
+                          return_lse: bool = False):
+    """Rank `rank`'s attention output for its zigzag query chunk; kv_chunks[r] = (k, v) of rank r, each
+    [batch, kv_heads, local_seq, head_dim] in rank r's zigzag order.  Differentiable w.r.t. q and every chunk."""
+    if len(kv_chunks) != world_size:
+        raise ValueError(f"need one K/V chunk per rank ({world_size}), got {len(kv_chunks)}")
+    flat: list[torch.Tensor] = []
+    for k, v in kv_chunks:
+        flat += [k, v]
+    out, lse = _ZigzagRingFunction.apply(q, rank, world_size, *flat)
+    return (out, lse) if return_lse else out
+
+
+class HipRingAttentionCore(nn.Module):
+    """`attn_core` drop-in (q, k, v, position_offset, position_ids, sequence_ids) -> out.
+
+    With world_size == 1 it is plain local attention, as the reference's core is
+    (runtime/layers/ring_attention.py:45-54).  With world_size > 1 the caller supplies
+    `kv_source(rank, k_local, v_local) -> [(k, v) for every rank]`, the seam where a transport plugs in.
+    """
+
+    preserves_native_gqa = True
+
+    def __init__(self, *, rank: int = 0, world_size: int = 1,
+                 kv_source: Callable[[int, torch.Tensor, torch.Tensor], Sequence[KvChunk]] | None = None,
+                 attention_backend: str = AttentionBackend.HIP) -> None:
+        super().__init__()
+        self.attention_backend = validate_attention_backend(attention_backend)
+        if world_size > 1 and kv_source is None:
+            raise ValueError("HipRingAttentionCore with world_size > 1 needs a kv_source")
+        self.rank, self.world_size, self.kv_source = rank, world_size, kv_source
+
+    def forward(self, q, k, v, position_offset: int, position_ids=None, sequence_ids=None) -> torch.Tensor:
+        if self.world_size == 1:
+            positions = canonical_position_ids(position_ids, batch_size=q.size(0), seq_len=q.size(-2),
+                                               position_offset=position_offset, device=q.device)
+            sequences = canonical_sequence_ids(sequence_ids, batch_size=q.size(0), seq_len=q.size(-2), device=q.device)
+            return causal_attention(q, k, v, attention_backend=self.attention_backend, warning_prefix="HipRingAttentionCore",
+                                    q_positions=positions, k_positions=positions, q_sequence_ids=sequences,
+                                    k_sequence_ids=sequences)
+        if sequence_ids is not None:
+            raise NotImplementedError("packed-document ring attention (varlen-prefix blocks) is not built yet")
+        chunks = self.kv_source(self.rank, k, v)
+        return zigzag_ring_attention(q, chunks, rank=self.rank, world_size=self.world_size)
