@@ -54,8 +54,8 @@ def hip_fallback_reason(q: torch.Tensor) -> str | None:
         return "the HIP attention kernels require GPU tensors"
     if q.dtype not in (torch.bfloat16, torch.float32):
         return f"the HIP attention kernels take bfloat16 or float32 tensors, got {q.dtype}"
-    if q.size(-1) > 256:
-        return f"head_dim {q.size(-1)} > 256 is not supported"
+    if q.size(-1) > 192:
+        return f"head_dim {q.size(-1)} > 192 is not supported"
     return None
 
 

@@ -29,7 +29,7 @@ const char* shape_problem(const mlts_attn_shape* s) {
   if (s->dtype != MLTS_BF16 && s->dtype != MLTS_F32) return "dtype must be MLTS_F32 or MLTS_BF16";
   if (s->B < 0 || s->Hq <= 0 || s->Hkv <= 0 || s->Sq < 0 || s->Sk < 0 || s->D <= 0) return "negative or zero dimension";
   if (s->Hq % s->Hkv != 0) return "Hq must be a multiple of Hkv";
-  if (s->D > 256) return "head_dim > 256 is not supported";
+  if (s->D > 192) return "head_dim > 192 is not supported";
   if (s->mask_mode < MLTS_MASK_NONE || s->mask_mode > MLTS_MASK_DOC) return "unknown mask_mode";
   if (!(s->scale > 0.f)) return "softmax scale must be positive";
   if (s->mask_mode == MLTS_MASK_DOC && !(s->q_pos && s->k_pos && s->q_seq && s->k_seq))
@@ -119,12 +119,16 @@ __global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc,
     pb = isfinite(lb) ? expf(lb - ln) : 0.f;
   }
   const T* bp = o_blk + b * bs0 + h * bs1 + static_cast<int64_t>(i) * bs2;
-  for (int vc = sub; vc < vec_per_row; vc += G) {
-    const f32x4 acc = reinterpret_cast<const f32x4*>(out_acc + arow * D)[vc];
-    f32x4 r;
+  if ((D & 3) == 0) {
+    for (int vc = sub; vc < vec_per_row; vc += G) {
+      const f32x4 acc = reinterpret_cast<const f32x4*>(out_acc + arow * D)[vc];
+      f32x4 r;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) r[e] = acc[e] * pa + to_f32<T>(bp[vc * 4 + e]) * pb;
-    reinterpret_cast<f32x4*>(out_acc + arow * D)[vc] = r;
+      for (int e = 0; e < 4; ++e) r[e] = acc[e] * pa + to_f32<T>(bp[vc * 4 + e]) * pb;
+      reinterpret_cast<f32x4*>(out_acc + arow * D)[vc] = r;
+    }
+  } else {
+    for (int d = sub; d < D; d += G) out_acc[arow * D + d] = out_acc[arow * D + d] * pa + to_f32<T>(bp[d]) * pb;
   }
   if (sub == 0) lse_acc[arow] = ln;
 }
@@ -223,14 +227,13 @@ extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk
   MLTS_REQUIRE(blk_dtype == MLTS_BF16 || blk_dtype == MLTS_F32, "mlts_attn_merge: unknown dtype %d", blk_dtype);
   MLTS_REQUIRE(B >= 0 && H >= 0 && S >= 0 && D > 0 && q_off >= 0 && q_len >= 0 && q_off + q_len <= S,
                "mlts_attn_merge: rows [%d, %d) do not fit S=%d", q_off, q_off + q_len, S);
-  MLTS_REQUIRE(D % 4 == 0, "mlts_attn_merge: head_dim must be a multiple of 4");
   if (B == 0 || H == 0 || q_len == 0) return MLTS_OK;
   MLTS_REQUIRE(out_acc && lse_acc && o_blk && lse_blk && o_blk_stride, "mlts_attn_merge: null pointer");
-  MLTS_REQUIRE(mlts_aligned16(out_acc), "mlts_attn_merge: out_acc must be 16-byte aligned");
+  MLTS_REQUIRE((D & 3) != 0 || mlts_aligned16(out_acc), "mlts_attn_merge: out_acc must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total_rows = static_cast<int64_t>(B) * H * q_len;
   int G = 1;
-  while (G < D / 4 && G < 64) G <<= 1;
+  while (G < (D + 3) / 4 && G < 64) G <<= 1;
   const int rows_per_block = 256 / G;
   const int64_t blocks = (total_rows + rows_per_block - 1) / rows_per_block;
   if (blk_dtype == MLTS_BF16)

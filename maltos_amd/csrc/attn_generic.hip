@@ -1,4 +1,4 @@
-// Generic attention kernels: any head_dim <= 256, fp32 or bf16 storage, fp32 arithmetic on the
+// Generic attention kernels: any head_dim <= 192, fp32 or bf16 storage, fp32 arithmetic on the
 // vector ALU (no MFMA).  They serve the fp32 configurations (1e-4 parity with the fp32 reference)
 // and head dims the MFMA kernels do not cover.  Structure: a workgroup owns 16 query rows (forward,
 // dQ) or 16 key rows (dK/dV) and walks the other side in tiles of 64 staged in LDS; in the score

@@ -4,6 +4,11 @@
 // are the reference's values and not merely close to them.
 #include "common.hpp"
 
+// The kernels below reproduce the reference's per-op bf16 roundings.  With contraction enabled the
+// compiler narrows "round(a * b)" to a bf16 multiply and then fuses it into the following add as an
+// fp32 FMA, which silently drops that rounding; contraction stays off for this whole file.
+#pragma clang fp contract(off)
+
 namespace {
 
 constexpr int kThreads = 256;

@@ -1,0 +1,299 @@
+"""GPU parity of the attention kernels (called through the torch.library ops -> C ABI) against the CPU
+oracle on identical seeded inputs: forward O and LSE, backward dQ/dK/dV, the LSE merge, the
+kernel-shaped flash_* function set and the zigzag ring schedule.
+
+Tolerances
+  * float32 (generic kernels) : 1e-4 relative (stated fp32 bar) with a 1e-5 absolute floor.
+  * bfloat16 (MFMA kernels)   : inputs are rounded to bf16 first and the oracle runs in fp32 on those values.
+      O, dQ, dK, dV : |err| <= 2e-2 + 2^-8 |want|.  2e-2 is the stated max-abs bar; the second term is half a
+                      bf16 ulp of the expected value, the rounding any bf16 output carries (it matters only
+                      for |want| > ~5, e.g. dV rows that sum many queries).
+      LSE (fp32)    : 2e-3 absolute.
+  * reference ring test vectors (fp32, head_dim 3): forward 1e-5, backward 2e-5, the reference's own bars.
+"""
+import pytest
+import torch
+
+from maltos_amd import ops
+from maltos_amd.attention_backend import causal_attention
+from maltos_amd.flash_utils import (flash_attn_dense, flash_attn_dense_backward, flash_attn_dense_with_lse,
+                                    flash_attn_varlen)
+from maltos_amd.llama import HipAttentionCore
+from maltos_amd.ring_attention import HipRingAttentionCore, zigzag_ring_attention
+from maltos_amd.ring_layout import expected_zigzag_ring_positions
+from oracle import attention as oa
+
+pytestmark = pytest.mark.gpu
+
+
+def check(got: torch.Tensor, want: torch.Tensor, dtype, what: str = "") -> None:
+    got, want = got.float().cpu(), want.float().cpu()
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    err = (got - want).abs()
+    bound = 1e-4 * want.abs() + 1e-5 if dtype == torch.float32 else 2e-2 + 2.0 ** -8 * want.abs()
+    assert (err <= bound).all(), f"{what}: worst excess {(err - bound).max().item():.3e} (max err {err.max().item():.3e})"
+
+
+def make_docs(B, S, gen, max_len, pad_tail=0):
+    pos = torch.zeros(B, S, dtype=torch.long)
+    seq = torch.full((B, S), -1, dtype=torch.long)
+    for b in range(B):
+        i = d = 0
+        while i < S - pad_tail:
+            L = min(int(torch.randint(1, max_len + 1, (1,), generator=gen)), S - pad_tail - i)
+            pos[b, i:i + L] = torch.arange(L)
+            seq[b, i:i + L] = d
+            i, d = i + L, d + 1
+    return pos, seq
+
+
+def bshd(B, H, S, D, gen, dtype):
+    return torch.randn(B, S, H, D, generator=gen).to(dtype).transpose(1, 2)
+
+
+def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad_tail=0):
+    gen = torch.Generator().manual_seed(seed)
+    q, k, v, do = bshd(B, Hq, Sq, D, gen, dtype), bshd(B, Hkv, Sk, D, gen, dtype), bshd(B, Hkv, Sk, D, gen, dtype), bshd(B, Hq, Sq, D, gen, dtype)
+    kw, mask = {}, None
+    if mode == ops.MASK_CAUSAL:
+        mask = oa.causal_mask(Sq, Sk, "cpu")
+    elif mode == ops.MASK_DOC:
+        assert Sq == Sk
+        pos, seq = make_docs(B, Sq, gen, max_doc or max(2, Sq // 3), pad_tail)
+        mask = oa.doc_mask(pos, pos, seq, seq)
+        kw = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+    qf, kf, vf = (t.detach().float().clone().requires_grad_(True) for t in (q, k, v))
+    want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
+    want_o.backward(do.float())
+    qg, kg, vg = (t.detach().to(dev).requires_grad_(True) for t in (q, k, v))
+    o, lse = ops.attention(qg, kg, vg, mask_mode=mode, return_lse=True, **kw)
+    o.backward(do.to(dev))
+    tag = f"dtype={dtype} B{B} Hq{Hq} Hkv{Hkv} Sq{Sq} Sk{Sk} D{D} mode{mode}"
+    check(o, want_o, dtype, tag + " O")
+    fin = torch.isfinite(want_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin), tag + " LSE -inf pattern"
+    lse_tol = 1e-4 if dtype == torch.float32 else 2e-3
+    assert (lse.cpu()[fin] - want_lse[fin]).abs().max() <= lse_tol, tag + " LSE"
+    check(qg.grad, qf.grad, dtype, tag + " dQ")
+    check(kg.grad, kf.grad, dtype, tag + " dK")
+    check(vg.grad, vf.grad, dtype, tag + " dV")
+    # explicit FlashAttention-2 backward of the oracle agrees too (pins the formula the kernel implements)
+    edq, edk, edv = oa.attention_backward_explicit(do, q, k, v, want_o.detach(), want_lse.detach(), mask)
+    check(qg.grad, edq, dtype, tag + " dQ(explicit)")
+    return o, lse
+
+
+CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, mode
+    (1, 1, 1, 1, 1, 64, ops.MASK_CAUSAL),
+    (2, 4, 4, 100, 100, 64, ops.MASK_CAUSAL),
+    (1, 2, 2, 256, 256, 128, ops.MASK_CAUSAL),
+    (2, 3, 3, 300, 300, 64, ops.MASK_CAUSAL),
+    (1, 4, 2, 515, 515, 128, ops.MASK_CAUSAL),
+    (1, 2, 1, 200, 333, 128, ops.MASK_NONE),
+    (1, 2, 2, 333, 200, 64, ops.MASK_NONE),
+    (1, 2, 2, 96, 224, 128, ops.MASK_CAUSAL),  # rectangular, bottom-right aligned
+    (2, 4, 2, 515, 515, 128, ops.MASK_DOC),
+    (2, 8, 2, 260, 260, 64, ops.MASK_DOC),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B{}_Hq{}_Hkv{}_Sq{}_Sk{}_D{}_m{}".format(*c))
+def test_forward_backward_parity(dev, dtype, case):
+    run_case(dev, dtype, *case, seed=sum(case))
+
+
+@pytest.mark.parametrize("D", [1, 3, 24, 96, 192])
+def test_generic_head_dims(dev, D):
+    run_case(dev, torch.float32, 1, 2, 1, 70, 70, D, ops.MASK_CAUSAL, seed=D)
+    if D % 8 == 0:
+        run_case(dev, torch.bfloat16, 1, 2, 2, 70, 70, D, ops.MASK_DOC, seed=D + 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_padding_rows_give_zeros_and_no_nan(dev, dtype):
+    o, lse = run_case(dev, dtype, 2, 2, 2, 200, 200, 64, ops.MASK_DOC, seed=77, max_doc=50, pad_tail=37)
+    assert not o[:, :, -37:].any() and (lse[:, :, -37:] == float("-inf")).all()
+
+
+def test_reference_known_answers_through_hip(dev, known_answers):
+    col = lambda vals: torch.tensor(vals, dtype=torch.float32, device=dev).view(1, 1, -1, 1)
+    ka = known_answers["packed_doc_attention"]
+    out = HipAttentionCore()(col(ka["q"]), col(ka["k"]), col(ka["v"]), 0, torch.tensor([ka["position_ids"]]),
+                             torch.tensor([ka["sequence_ids"]]))
+    assert torch.allclose(out.flatten().cpu(), torch.tensor(ka["expected"]), atol=ka["atol"])
+    kc = known_answers["cross_chunk_attention"]
+    ids = lambda key: torch.tensor([kc[key]], device=dev)
+    out = causal_attention(col(kc["q"]), col(kc["k"]), col(kc["v"]), attention_backend="hip", warning_prefix="test",
+                           q_positions=ids("q_positions"), k_positions=ids("k_positions"),
+                           q_sequence_ids=ids("q_sequence_ids"), k_sequence_ids=ids("k_sequence_ids"),
+                           flash_varlen_mode="prefix")
+    assert torch.allclose(out.flatten().cpu(), torch.tensor(kc["expected"]), atol=kc["atol"])
+
+
+def test_hip_backend_agrees_with_sdpa_backend_on_device(dev):
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = (bshd(2, 4, 129, 64, gen, torch.float32).to(dev) for _ in range(3))
+    a = causal_attention(q, k, v, attention_backend="hip", warning_prefix="t")
+    b = causal_attention(q, k, v, attention_backend="sdpa_auto", warning_prefix="t")
+    assert torch.allclose(a, b, atol=1e-5)
+    pos, seq = make_docs(2, 129, gen, 40)
+    kw = dict(q_positions=pos.to(dev), k_positions=pos.to(dev), q_sequence_ids=seq.to(dev), k_sequence_ids=seq.to(dev))
+    a = causal_attention(q, k, v, attention_backend="hip", warning_prefix="t", **kw)
+    b = causal_attention(q, k, v, attention_backend="eager", warning_prefix="t", **kw)
+    assert torch.allclose(a, b, atol=1e-5)
+
+
+def test_empty_and_error_cases(dev):
+    z = torch.zeros(0, 2, 8, 64, device=dev, dtype=torch.bfloat16)
+    o, lse = ops.attention_forward(z, z, z, mask_mode=ops.MASK_CAUSAL)
+    assert o.shape == (0, 2, 8, 64) and lse.shape == (0, 2, 8)
+    q = torch.randn(1, 2, 0, 64, device=dev)
+    kv = torch.randn(1, 2, 5, 64, device=dev)
+    o, lse = ops.attention_forward(q, kv, kv, mask_mode=ops.MASK_NONE)
+    assert o.shape == (1, 2, 0, 64)
+    q = torch.randn(1, 2, 4, 64, device=dev)
+    o, lse = ops.attention_forward(q, kv[:, :, :0], kv[:, :, :0], mask_mode=ops.MASK_NONE)  # no keys: zeros, -inf
+    assert not o.any() and (lse == float("-inf")).all()
+    with pytest.raises(ValueError):
+        ops.attention(q, kv.half(), kv.half())
+    with pytest.raises(ValueError):
+        ops.attention(q, kv, kv, mask_mode=ops.MASK_DOC)  # ids missing
+    with pytest.raises(ValueError):
+        ops.attention(torch.randn(1, 1, 4, 300, device=dev), torch.randn(1, 1, 4, 300, device=dev), torch.randn(1, 1, 4, 300, device=dev))
+
+
+@pytest.mark.parametrize("D,blk_dtype", [(128, torch.bfloat16), (64, torch.float32), (3, torch.float32)])
+def test_merge_kernel(dev, D, blk_dtype):
+    gen = torch.Generator().manual_seed(D)
+    B, H, S = 2, 3, 50
+    ro = torch.randn(B, H, S, D, generator=gen)
+    rl = torch.randn(B, H, S, generator=gen)
+    rl[0, 0, :5] = float("-inf")
+    ro[0, 0, :5] = 0
+    bo = torch.randn(B, S, H, D, generator=gen).to(blk_dtype).transpose(1, 2)
+    bl = torch.randn(B, H, S, generator=gen)
+    bl[0, 0, 3:8] = float("-inf")
+    want_o, want_l = oa.merge_attention_blocks(ro.clone(), rl.clone(), bo, bl)
+    go, gl = ro.to(dev), rl.to(dev)
+    ops.attention_merge_(go, gl, bo.to(dev), bl.to(dev), 0)
+    torch.testing.assert_close(go.cpu(), want_o, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gl.cpu(), want_l, rtol=1e-5, atol=1e-6)
+    # slice form
+    want_o2, want_l2 = ro.clone(), rl.clone()
+    oa.merge_attention_blocks(want_o2, want_l2, bo[:, :, :20], bl[:, :, :20], q_slice=slice(30, None))
+    go, gl = ro.to(dev), rl.to(dev)
+    ops.attention_merge_(go, gl, bo[:, :, :20].to(dev), bl[:, :, :20].contiguous().to(dev), 30)
+    torch.testing.assert_close(go.cpu(), want_o2, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gl.cpu(), want_l2, rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        ops.attention_merge_(go, gl, bo[:, :, :20].to(dev), bl[:, :, :20].contiguous().to(dev), 40)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_block_functions_compose_with_global_lse(dev, dtype):
+    """Two key blocks merged == one pass; block backwards fed the GLOBAL out/LSE sum to the full backward."""
+    gen = torch.Generator().manual_seed(9)
+    B, H, S, D = 1, 2, 192, 64
+    q, k, v, do = (bshd(B, H, S, D, gen, dtype).to(dev) for _ in range(4))
+    full = flash_attn_dense_with_lse(q, k, v, causal=False)
+    a = flash_attn_dense_with_lse(q, k[:, :, :64], v[:, :, :64], causal=False)
+    b = flash_attn_dense_with_lse(q, k[:, :, 64:], v[:, :, 64:], causal=False)
+    ro = torch.zeros(B, H, S, D, device=dev)
+    rl = torch.full((B, H, S), float("-inf"), device=dev)
+    ops.attention_merge_(ro, rl, a.out, a.lse)
+    ops.attention_merge_(ro, rl, b.out, b.lse)
+    check(ro, full.out, dtype, "merged O")
+    assert (rl - full.lse).abs().max() <= (1e-5 if dtype == torch.float32 else 2e-3)
+    dq, dk, dv = flash_attn_dense_backward(do, q, k, v, full.out, full.lse, causal=False)
+    dq1, dk1, dv1 = flash_attn_dense_backward(do, q, k[:, :, :64], v[:, :, :64], full.out, full.lse, causal=False)
+    dq2, dk2, dv2 = flash_attn_dense_backward(do, q, k[:, :, 64:], v[:, :, 64:], full.out, full.lse, causal=False)
+    check(dq1.float() + dq2.float(), dq, dtype, "dQ sum")
+    check(torch.cat([dk1, dk2], 2), dk, dtype, "dK cat")
+    check(torch.cat([dv1, dv2], 2), dv, dtype, "dV cat")
+    want_o, want_lse = oa.attention_with_lse(q.cpu(), k.cpu(), v.cpu())
+    check(full.out, want_o, dtype, "block O vs oracle")
+    # differentiable dense causal entry point
+    qg = q.clone().requires_grad_(True)
+    flash_attn_dense(qg, k, v).backward(do)
+    rq = q.cpu().float().requires_grad_(True)
+    oa.attention_with_lse(rq, k.cpu(), v.cpu(), oa.causal_mask(S, S, "cpu"))[0].backward(do.cpu().float())
+    check(qg.grad, rq.grad, dtype, "flash_attn_dense dQ")
+
+
+def test_flash_attn_varlen_runs_and_padding(dev):
+    gen = torch.Generator().manual_seed(13)
+    ids = torch.tensor([[0, 0, 0, 1, 1, -1, 0, 0], [2, 2, 3, 3, 3, 3, -1, -1]])  # id 0 appears in two separate runs
+    q, k, v = (bshd(2, 2, 8, 64, gen, torch.float32) for _ in range(3))
+    out = flash_attn_varlen(q.to(dev), k.to(dev), v.to(dev), ids.to(dev)).cpu()
+    runs = torch.tensor([[0, 0, 0, 1, 1, -1, 2, 2], [0, 0, 1, 1, 1, 1, -1, -1]])
+    idx = torch.arange(8).unsqueeze(0).expand(2, -1)
+    want, _ = oa.attention_with_lse(q, k, v, oa.doc_mask(idx, idx, runs, runs))
+    assert torch.allclose(out, want, atol=1e-5)
+    assert not out[0, :, 5].any() and not out[1, :, 6:].any()
+
+
+def _ring_inputs(world_size, s_loc, B, H, D, dtype, seeds):
+    total = s_loc * world_size
+    mk = lambda s: torch.randn((B, H, total, D), generator=torch.Generator().manual_seed(s + world_size)).to(dtype)
+    all_q, all_k, all_v = mk(seeds["q"]), mk(seeds["k"]), mk(seeds["v"])
+    pos = [expected_zigzag_ring_positions(s_loc, rank=r, world_size=world_size, device=torch.device("cpu")) for r in range(world_size)]
+    pick = lambda t: [t.index_select(2, p) for p in pos]
+    return all_q, all_k, all_v, pos, pick(all_q), pick(all_k), pick(all_v)
+
+
+@pytest.mark.parametrize("world_size", [2, 4])
+def test_zigzag_ring_reference_vectors_fp32(dev, known_answers, world_size):
+    spec = known_answers["zigzag_ring_schedule"]
+    all_q, all_k, all_v, pos, qc, kc, vc = _ring_inputs(world_size, spec["local_seq_len"], spec["batch"], spec["heads"],
+                                                        spec["head_dim"], torch.float32, spec["seed_offsets"])
+    total = spec["local_seq_len"] * world_size
+    gq, gk, gv = (t.clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, glse = oa.attention_with_lse(gq, gk, gv, oa.causal_mask(total, total, "cpu"))
+    dout_all = torch.randn(gout.shape, generator=torch.Generator().manual_seed(99))
+    gout.backward(dout_all)
+    dk_sum, dv_sum = torch.zeros_like(all_k), torch.zeros_like(all_v)
+    for rank in range(world_size):
+        q = qc[rank].to(dev).requires_grad_(True)
+        chunks = [(k.to(dev).requires_grad_(True), v.to(dev).requires_grad_(True)) for k, v in zip(kc, vc)]
+        out, lse = zigzag_ring_attention(q, chunks, rank=rank, world_size=world_size, return_lse=True)
+        assert torch.allclose(out.cpu(), gout.detach().index_select(2, pos[rank]), atol=spec["forward_atol"])
+        assert torch.allclose(lse.cpu(), glse.detach().index_select(2, pos[rank]), atol=spec["forward_atol"])
+        out.backward(dout_all.index_select(2, pos[rank]).to(dev))
+        assert torch.allclose(q.grad.cpu(), gq.grad.index_select(2, pos[rank]), atol=spec["backward_atol"])
+        for src, (k, v) in enumerate(chunks):
+            dk_sum.index_add_(2, pos[src], k.grad.cpu())
+            dv_sum.index_add_(2, pos[src], v.grad.cpu())
+    assert torch.allclose(dk_sum, gk.grad, atol=spec["backward_atol"])
+    assert torch.allclose(dv_sum, gv.grad, atol=spec["backward_atol"])
+
+
+def test_zigzag_ring_bf16_matches_global_causal(dev):
+    world_size, s_loc, B, H, D = 4, 256, 1, 2, 128
+    all_q, all_k, all_v, pos, qc, kc, vc = _ring_inputs(world_size, s_loc, B, H, D, torch.bfloat16, dict(q=1, k=2, v=3))
+    total = s_loc * world_size
+    gq, gk, gv = (t.detach().float().clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, glse = oa.attention_with_lse(gq, gk, gv, oa.causal_mask(total, total, "cpu"))
+    dout_all = torch.randn(gout.shape, generator=torch.Generator().manual_seed(7)).bfloat16()
+    gout.backward(dout_all.float())
+    dk_sum, dv_sum = torch.zeros_like(gk.grad), torch.zeros_like(gv.grad)
+    for rank in range(world_size):
+        q = qc[rank].to(dev).requires_grad_(True)
+        chunks = [(k.to(dev).requires_grad_(True), v.to(dev).requires_grad_(True)) for k, v in zip(kc, vc)]
+        core = HipRingAttentionCore(rank=rank, world_size=world_size, kv_source=lambda r, k, v, c=chunks: c)
+        out = core(q, chunks[rank][0], chunks[rank][1], 0, pos[rank])
+        check(out, gout.detach().index_select(2, pos[rank]), torch.bfloat16, f"ring O rank{rank}")
+        out.backward(dout_all.index_select(2, pos[rank]).to(dev))
+        check(q.grad, gq.grad.index_select(2, pos[rank]), torch.bfloat16, f"ring dQ rank{rank}")
+        for src, (k, v) in enumerate(chunks):
+            if k.grad is not None:
+                dk_sum.index_add_(2, pos[src], k.grad.float().cpu())
+                dv_sum.index_add_(2, pos[src], v.grad.float().cpu())
+    # each chunk's dK/dV is the sum of four bf16-rounded rank contributions
+    assert ((dk_sum - gk.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gk.grad.abs())).all()
+    assert ((dv_sum - gv.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gv.grad.abs())).all()
+    # world_size == 1 degenerates to plain causal attention
+    solo = HipRingAttentionCore()(all_q[:, :, :256].to(dev), all_k[:, :, :256].to(dev), all_v[:, :, :256].to(dev), 0)
+    want, _ = oa.attention_with_lse(all_q[:, :, :256], all_k[:, :, :256], all_v[:, :, :256], oa.causal_mask(256, 256, "cpu"))
+    check(solo, want, torch.bfloat16, "single-rank ring")

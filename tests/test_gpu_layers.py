@@ -1,0 +1,197 @@
+"""GPU parity of the HBM-bound kernels (through the torch.library ops, i.e. through the C ABI) against
+the CPU oracle on identical seeded inputs.
+
+Tolerances:
+  * fp32                : 1e-4 relative (the stated fp32 bar); most agree to ~1e-6.
+  * bf16 forward        : RMSNorm / RoPE / SwiGLU reproduce the reference's eager roundings, so they are
+                          compared to the oracle's bf16 evaluation and may differ by at most one bf16 ulp
+                          (rsqrt/exp differ in the last fp32 bit between CPU and GPU) on < 0.1 % of entries.
+  * bf16 backward, loss : fp32 math inside the kernel and ONE rounding of the result, so against the oracle's
+                          fp32 formulas on the bf16-rounded inputs |err| <= 2^-8 |want| + 1e-3 (half a bf16 ulp);
+                          loss 1e-4 relative (it is returned in fp32).
+"""
+import pytest
+import torch
+
+from maltos_amd import ops
+from oracle import layers as ol
+from oracle import optim as oo
+
+pytestmark = pytest.mark.gpu
+
+
+def _one_rounding(got: torch.Tensor, want: torch.Tensor) -> None:
+    """fp32 math + a single bf16 rounding of the result: |err| <= 2^-8 |want| (half an ulp) + 1e-3."""
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs()
+    bound = 2.0 ** -8 * want.abs() + 1e-3
+    assert (err <= bound).all(), f"worst excess {(err - bound).max().item()}"
+
+
+def _ulp_close(got: torch.Tensor, want: torch.Tensor, max_frac: float = 1e-3) -> None:
+    got, want = got.float().cpu(), want.float().cpu()
+    diff = (got - want).abs()
+    ulp = torch.maximum(want.abs(), torch.tensor(1e-30)) * 2.0 ** -7  # one bf16 ulp is <= 2^-7 relative
+    assert (diff <= ulp).all(), f"max diff {diff.max().item()} exceeds one bf16 ulp"
+    assert (diff > 0).float().mean().item() <= max_frac, "too many entries differ from the oracle's rounding"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden", [(1, 256), (37, 512), (300, 1024)])
+def test_rmsnorm_forward_backward(dev, dtype, rows, hidden):
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = torch.randn(rows, hidden, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    dy = torch.randn(rows, hidden, generator=g).to(dtype)
+    xg, wg = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    y = ops.rms_norm(xg, wg, 1e-5)
+    y.backward(dy.to(dev))
+    want = ol.rms_norm(x, w, 1e-5)
+    dx, dw = ol.rms_norm_backward(dy, x, w, 1e-5)
+    if dtype == torch.float32:
+        torch.testing.assert_close(y.cpu(), want, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(xg.grad.cpu(), dx, rtol=1e-4, atol=1e-5)
+        torch.testing.assert_close(wg.grad.cpu(), dw, rtol=1e-4, atol=1e-4)
+    else:
+        _ulp_close(y, want)
+        _one_rounding(xg.grad, dx)
+        assert ((wg.grad.float().cpu() - dw).abs() <= 2e-2 + 2.0 ** -8 * dw.abs()).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_ids", [False, True])
+def test_rope_forward_backward(dev, dtype, use_ids):
+    B, H, S, D = 2, 3, 17, 64
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(B, S, H, D, generator=g).to(dtype).transpose(1, 2)  # the [B,H,S,D] view LlamaAttention makes
+    dy = torch.randn(B, S, H, D, generator=g).to(dtype).transpose(1, 2)
+    cos_t, sin_t = ol.rope_tables(D, 64)
+    cos_t, sin_t = cos_t.to(dtype), sin_t.to(dtype)
+    pos = torch.stack([torch.arange(S) % 5, torch.arange(S) + 3]) if use_ids else None
+    cos, sin = ol.rope_cos_sin(cos_t, sin_t, seq_len=S, position_offset=4, position_ids=pos)
+    want = ol.apply_rotary(x, cos, sin)
+    want_dx = ol.apply_rotary_backward(dy, cos, sin)
+    xg = x.to(dev).requires_grad_(True)
+    y = ops.rope(xg, cos_t.to(dev), sin_t.to(dev), positions=None if pos is None else pos.to(dev), position_offset=4)
+    assert y.stride() == xg.stride()
+    y.backward(dy.to(dev))
+    if dtype == torch.float32:
+        torch.testing.assert_close(y.cpu(), want, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(xg.grad.cpu(), want_dx, rtol=1e-4, atol=1e-6)
+    else:  # every product and sum rounded where the reference's eager ops round: bit exact
+        assert torch.equal(y.cpu(), want)
+        assert torch.equal(xg.grad.cpu(), want_dx)
+    with pytest.raises(ValueError):
+        ops.rope(xg, cos_t.to(dev)[:8], sin_t.to(dev)[:8], position_offset=4)  # table too short
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n", [(5, 7), (64, 1376)])
+def test_swiglu_forward_backward(dev, dtype, n):
+    g = torch.Generator().manual_seed(sum(n))
+    gate = (2 * torch.randn(*n, generator=g)).to(dtype)
+    up = torch.randn(*n, generator=g).to(dtype)
+    dh = torch.randn(*n, generator=g).to(dtype)
+    gg, ug = gate.to(dev).requires_grad_(True), up.to(dev).requires_grad_(True)
+    h = ops.swiglu(gg, ug)
+    h.backward(dh.to(dev))
+    want = ol.swiglu(gate, up)
+    dg, du = ol.swiglu_backward(dh, gate, up)
+    if dtype == torch.float32:
+        torch.testing.assert_close(h.cpu(), want, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(gg.grad.cpu(), dg, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(ug.grad.cpu(), du, rtol=1e-4, atol=1e-6)
+    else:
+        _ulp_close(h, want)
+        _one_rounding(gg.grad, dg)
+        _one_rounding(ug.grad, du)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,vocab", [(6, 5), (64, 8192), (33, 32000), (5, 50257)])
+def test_cross_entropy(dev, dtype, rows, vocab):
+    g = torch.Generator().manual_seed(rows * vocab % 9973)
+    logits = (3 * torch.randn(rows, vocab, generator=g)).to(dtype)
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    labels[::3] = -100
+    lg = logits.to(dev).requires_grad_(True)
+    loss = ops.cross_entropy(lg, labels.to(dev))
+    assert loss.dtype == torch.float32
+    (loss * 1.0).backward()
+    want_loss, want_grad = ol.causal_cross_entropy_explicit(logits, labels)
+    assert abs(loss.item() - want_loss.item()) <= 1e-4 * abs(want_loss.item()) + 1e-6
+    tol = 1e-6 if dtype == torch.float32 else 2.0 ** -8
+    assert ((lg.grad.float().cpu() - want_grad).abs() <= tol * want_grad.abs() + 1e-7).all()
+    # upstream gradient other than one, and the reference's library form
+    lg2 = logits.to(dev).requires_grad_(True)
+    (ops.cross_entropy(lg2, labels.to(dev)) * 0.25).backward()
+    assert ((lg2.grad.float().cpu() - 0.25 * want_grad).abs() <= 2 * tol * want_grad.abs() + 1e-7).all()
+    lib = ol.causal_cross_entropy(logits.float(), labels)
+    assert abs(loss.item() - lib.item()) <= 1e-4 * abs(lib.item()) + 1e-6
+
+
+def test_cross_entropy_without_targets_is_zero(dev):
+    lg = torch.randn(2, 3, 5, device=dev, requires_grad=True)
+    loss = ops.cross_entropy(lg, torch.full((2, 3), -100, device=dev))
+    assert loss.item() == 0.0
+    loss.backward()
+    assert not lg.grad.any()
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 4099, 1 << 20])
+def test_adamw_steps_match_library_and_closed_form(dev, n):
+    g = torch.Generator().manual_seed(n)
+    p0 = torch.randn(n, generator=g)
+    hp = dict(lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    ref = torch.nn.Parameter(p0.clone())
+    lib = torch.optim.AdamW([ref], lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"], weight_decay=hp["weight_decay"])
+    p, m, v = p0.to(dev), torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+    lowp = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    cp, cm, cv = p0.clone(), torch.zeros(n), torch.zeros(n)
+    for step in (1, 2, 3):
+        grad = 0.01 * torch.randn(n, generator=g)
+        ref.grad = grad.clone()
+        lib.step()
+        ops.adamw_step_(p, grad.to(dev), m, v, step=step, p_lowp=lowp, **hp)
+        cp, cm, cv = oo.adamw_reference_step(cp, grad, cm, cv, step=step, **hp)
+        torch.testing.assert_close(p.cpu(), ref.detach(), rtol=1e-4, atol=1e-7)
+        torch.testing.assert_close(p.cpu(), cp, rtol=1e-4, atol=1e-7)
+        assert torch.equal(lowp.cpu(), p.cpu().bfloat16())
+    torch.testing.assert_close(m.cpu(), lib.state[ref]["exp_avg"], rtol=1e-4, atol=1e-9)
+    torch.testing.assert_close(v.cpu(), lib.state[ref]["exp_avg_sq"], rtol=1e-4, atol=1e-12)
+
+
+def test_adamw_on_unaligned_views_and_fused_clip(dev):
+    n = 1003
+    g = torch.Generator().manual_seed(3)
+    base = torch.randn(4 * n + 8, generator=g).to(dev)
+    p, grad, m, v = (base[1 + i * n: 1 + (i + 1) * n] for i in range(4))  # 4-byte aligned only
+    m.zero_(), v.zero_()
+    p0, g0 = p.cpu().clone(), grad.cpu().clone()
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.0)
+    sq = ops.sq_norm(grad.contiguous())
+    norm = float(sq.sqrt().item())
+    assert abs(norm - oo.global_grad_norm([g0])) <= 1e-6 * norm
+    ops.adamw_step_(p, grad, m, v, step=1, sq_norm=sq, max_norm=1.0, **hp)
+    coef = oo.clip_coefficient(norm, 1.0)
+    assert coef < 1.0
+    want, _, _ = oo.adamw_reference_step(p0, g0 * coef, torch.zeros(n), torch.zeros(n), step=1, **hp)
+    torch.testing.assert_close(p.cpu(), want, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("n", [3, 4096, 1234567])
+@pytest.mark.parametrize("src_dtype", [torch.bfloat16, torch.float32])
+def test_grad_to_f32_and_norm(dev, n, src_dtype):
+    g = torch.Generator().manual_seed(n)
+    src = torch.randn(n, generator=g).to(src_dtype)
+    dst = torch.full((n,), 7.0, device=dev)
+    sq = torch.zeros((), dtype=torch.float64, device=dev)
+    ops.grad_to_f32_(dst, src.to(dev), sq_out=sq)
+    assert torch.equal(dst.cpu(), src.float())
+    want = src.double().pow(2).sum().item()
+    assert abs(sq.item() - want) <= 1e-12 * want
+    ops.grad_to_f32_(dst, src.to(dev), accumulate=True)
+    assert torch.equal(dst.cpu(), src.float() * 2)
+    assert abs(ops.sq_norm(dst).item() - 4 * want) <= 1e-12 * 4 * want
+    ops.scale_(dst, 0.5)
+    assert torch.equal(dst.cpu(), src.float())
