@@ -1,0 +1,256 @@
+"""The five benchmark configurations on the GPU, at their real sizes, through the product path.
+
+Seeds: one CPU generator seeded with 1234 per configuration, tensors drawn in the order they are listed;
+low-precision inputs are drawn in fp32 and rounded, so oracle and kernels see identical bits.  At these
+sizes the oracle (plain PyTorch, fp32) is evaluated on the GPU tensor by tensor / head by head; it is the
+same code the CPU tests pin.
+
+Tolerances (also written next to each check):
+  cfg1 fp32      : loss, grad-norm and post-step parameters 1e-4 relative.
+  cfg2-4 bf16    : O, dQ, dK, dV |err| <= 2e-2 + 2^-8 |want|, LSE 2e-3 (see tests/test_gpu_attention.py).
+  cfg5 bf16 step : loss and grad-norm 1e-3 relative against the fp32 evaluation of the same bf16-rounded
+                   network, and the reference-style bf16 eager evaluation must sit within the same distance.
+"""
+import json
+import math
+from collections import OrderedDict
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from maltos_amd import ops
+from maltos_amd.grad_clip import clip_grad_norm_
+from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
+from maltos_amd.ring_attention import zigzag_ring_attention
+from maltos_amd.ring_layout import expected_zigzag_ring_positions
+from oracle import attention as oa
+from oracle import llama as ol
+from oracle import optim as oo
+from tests.conftest import GOLDEN_DIR
+from tests.golden.make_cfg1_fixture import cfg1_inputs
+
+pytestmark = pytest.mark.gpu
+SEED = 1234
+
+
+def check_bf16(got, want, what):
+    got, want = got.float(), want.float()
+    assert torch.isfinite(got).all(), what
+    err = (got - want).abs()
+    bound = 2e-2 + 2.0 ** -8 * want.abs()
+    assert (err <= bound).all(), f"{what}: worst excess {(err - bound).max().item():.3e}, max err {err.max().item():.3e}"
+    return err.max().item()
+
+
+def load_into(model, params):
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            p.copy_(params[name].to(p.dtype))
+
+
+# ------------------------------------------------------------------ cfg1
+def test_cfg1_tiny_llama_fp32_step(dev):
+    fixture = json.loads((GOLDEN_DIR / "cfg1_tiny_llama_step.json").read_text())
+    cfg, params, input_ids, labels = cfg1_inputs()
+    want_loss, want_norm, want_params = ol.train_step(params, cfg, input_ids, labels)  # CPU oracle, ~3 s
+    assert abs(want_loss - fixture["loss"]) <= 1e-4 * fixture["loss"]
+    model = LlamaForCausalLM(LlamaConfig(**fixture["config"])).to(dev)
+    load_into(model, params)
+    opt = FusedAdamW(model.parameters(), lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    loss = model({"input_ids": input_ids.to(dev), "labels": labels.to(dev)})
+    loss.backward()
+    grads = OrderedDict((n, p.grad.detach().cpu()) for n, p in model.named_parameters())
+    norm = oo.global_grad_norm(grads.values())
+    assert abs(loss.item() - want_loss) <= 1e-4 * want_loss, (loss.item(), want_loss)
+    assert abs(norm - want_norm) <= 1e-4 * want_norm, (norm, want_norm)
+    assert abs(norm - fixture["grad_norm"]) <= 1e-4 * fixture["grad_norm"]
+    opt.step()
+    for name, p in model.named_parameters():
+        got, want = p.detach().cpu(), want_params[name]
+        rel = (got - want).norm() / want.norm()
+        assert rel <= 1e-4, f"{name}: relative error {rel.item():.2e}"
+        # elementwise: AdamW's first step is lr * g / (|g| + eps), which amplifies fp32 noise only where |g| ~ eps
+        close = torch.isclose(got, want, rtol=1e-4, atol=1e-6)
+        assert close.float().mean().item() >= 0.9999, name
+        rec = fixture["params"][name]
+        assert abs(float(got.double().abs().sum()) - rec["abs_sum"]) <= 1e-4 * rec["abs_sum"], name
+
+
+# ------------------------------------------------------------------ cfg2
+def _sdpa_math_fp32(q, k, v, causal=True):
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    with sdpa_kernel(SDPBackend.MATH):
+        return F.scaled_dot_product_attention(q, k, v, is_causal=causal)
+
+
+def test_cfg2_dense_causal_bf16_full_size(dev):
+    B, H, S, D = 4, 16, 4096, 128
+    gen = torch.Generator().manual_seed(SEED)
+    q, k, v, do = (torch.randn(B, H, S, D, generator=gen).bfloat16().to(dev) for _ in range(4))
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o, lse = ops.attention(qg, kg, vg, mask_mode=ops.MASK_CAUSAL, return_lse=True)
+    o.backward(do)
+    worst = {}
+    mask = oa.causal_mask(S, S, dev)
+    for b in range(B):
+        qf, kf, vf = (t[b:b + 1].float().requires_grad_(True) for t in (q, k, v))
+        want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
+        want_o.backward(do[b:b + 1].float())
+        worst["O"] = max(worst.get("O", 0), check_bf16(o[b:b + 1], want_o, f"O[{b}]"))
+        assert (lse[b:b + 1] - want_lse).abs().max() <= 2e-3
+        worst["dQ"] = max(worst.get("dQ", 0), check_bf16(qg.grad[b:b + 1], qf.grad, f"dQ[{b}]"))
+        worst["dK"] = max(worst.get("dK", 0), check_bf16(kg.grad[b:b + 1], kf.grad, f"dK[{b}]"))
+        worst["dV"] = max(worst.get("dV", 0), check_bf16(vg.grad[b:b + 1], vf.grad, f"dV[{b}]"))
+        if b == 0:  # the library routine the configuration names
+            lib = _sdpa_math_fp32(qf.detach(), kf.detach(), vf.detach())
+            assert (lib - want_o).abs().max() <= 1e-5
+    print(f"cfg2 max abs errors: {worst}")
+    # size-independent invariants: softmax rows sum to one
+    ones = torch.ones_like(v)
+    o1 = ops.attention(q, k, ones, mask_mode=ops.MASK_CAUSAL)
+    assert (o1.float() - 1.0).abs().max() <= 2.0 ** -7
+    #   => sum over keys of dV equals sum over queries of dO, per head and channel
+    got = vg.grad.float().sum(dim=2)
+    want = do.float().sum(dim=2)
+    assert (got - want).abs().max() <= 2e-2 * math.sqrt(S) + 2.0 ** -8 * want.abs().max()
+    #   causality: outputs of the first half do not depend on the second half of K/V
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, S // 2:] = 0
+    v2[:, :, S // 2:] = 7
+    o2 = ops.attention(q, k2, v2, mask_mode=ops.MASK_CAUSAL)
+    assert torch.equal(o2[:, :, :S // 2], o[:, :, :S // 2])
+
+
+# ------------------------------------------------------------------ cfg3
+def _packed_rows(B, S, gen):
+    pos = torch.zeros(B, S, dtype=torch.long)
+    seq = torch.zeros(B, S, dtype=torch.long)
+    docs = []
+    for b in range(B):
+        i = d = 0
+        row = []
+        while i < S:
+            L = min(int(torch.randint(64, 2049, (1,), generator=gen)), S - i)
+            pos[b, i:i + L] = torch.arange(L)
+            seq[b, i:i + L] = d
+            row.append((i, L))
+            i, d = i + L, d + 1
+        docs.append(row)
+    return pos, seq, docs
+
+
+def test_cfg3_packed_documents_gqa_bf16_full_size(dev):
+    B, S, Hq, Hkv, D = 2, 8192, 32, 8, 128
+    gen = torch.Generator().manual_seed(SEED)
+    pos, seq, docs = _packed_rows(B, S, gen)
+    q = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    k = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    v = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    do = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ids = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+    o, lse = ops.attention(qg, kg, vg, mask_mode=ops.MASK_DOC, return_lse=True, **ids)
+    o.backward(do)
+    work = 0
+    for b in range(B):
+        for start, L in docs[b]:
+            sl = slice(start, start + L)
+            qf, kf, vf = (t[b:b + 1, :, sl].float().requires_grad_(True) for t in (q, k, v))
+            want_o, want_lse = oa.attention_with_lse(qf, kf, vf, oa.causal_mask(L, L, dev))  # K/V head = h // 4
+            want_o.backward(do[b:b + 1, :, sl].float())
+            check_bf16(o[b:b + 1, :, sl], want_o, f"O[{b},{start}]")
+            assert (lse[b:b + 1, :, sl] - want_lse).abs().max() <= 2e-3
+            check_bf16(qg.grad[b:b + 1, :, sl], qf.grad, f"dQ[{b},{start}]")
+            check_bf16(kg.grad[b:b + 1, :, sl], kf.grad, f"dK[{b},{start}]")  # summed over the 4-head group
+            check_bf16(vg.grad[b:b + 1, :, sl], vf.grad, f"dV[{b},{start}]")
+            work += L * L // 2
+    print(f"cfg3 documents per row: {[len(d) for d in docs]}, score elements/head: {work}")
+
+
+# ------------------------------------------------------------------ cfg4
+@pytest.mark.parametrize("rank", [0, 2])
+def test_cfg4_zigzag_ring_rank_share_bf16_full_size(dev, rank):
+    W, H, S_loc, D = 4, 16, 8192, 128
+    total = W * S_loc
+    gen = torch.Generator().manual_seed(SEED)
+    gq, gk, gv, gdo = (torch.randn(1, H, total, D, generator=gen).bfloat16().to(dev) for _ in range(4))
+    pos = [expected_zigzag_ring_positions(S_loc, rank=r, world_size=W, device=dev) for r in range(W)]
+    q = gq.index_select(2, pos[rank]).requires_grad_(True)
+    chunks = [(gk.index_select(2, p).requires_grad_(True), gv.index_select(2, p).requires_grad_(True)) for p in pos]
+    out, lse = zigzag_ring_attention(q, chunks, rank=rank, world_size=W, return_lse=True)
+    out.backward(gdo.index_select(2, pos[rank]))
+    # oracle: ONE pass of causal attention over all 32768 tokens, head by head, with dO zero outside this rank
+    do_masked = torch.zeros_like(gdo)
+    do_masked[:, :, pos[rank]] = gdo[:, :, pos[rank]]
+    mask = oa.causal_mask(total, total, dev)
+    for h in range(H):
+        qf, kf, vf = (t[:, h:h + 1].float().requires_grad_(True) for t in (gq, gk, gv))
+        want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
+        want_o.backward(do_masked[:, h:h + 1].float())
+        check_bf16(out[:, h:h + 1], want_o.detach()[:, :, pos[rank]], f"O head {h}")
+        assert (lse[:, h:h + 1] - want_lse.detach()[:, :, pos[rank]]).abs().max() <= 2e-3
+        check_bf16(q.grad[:, h:h + 1], qf.grad[:, :, pos[rank]], f"dQ head {h}")
+        for src, (kc, vc) in enumerate(chunks):
+            check_bf16(kc.grad[:, h:h + 1], kf.grad[:, :, pos[src]], f"dK head {h} chunk {src}")
+            check_bf16(vc.grad[:, h:h + 1], vf.grad[:, :, pos[src]], f"dV head {h} chunk {src}")
+        del qf, kf, vf, want_o, want_lse
+
+
+# ------------------------------------------------------------------ cfg5
+CFG5 = dict(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8, num_attention_heads=8,
+            max_position_embeddings=2048, rms_norm_eps=1e-5, rope_theta=10000.0)
+
+
+def cfg5_inputs():
+    cfg = ol.OracleLlamaConfig(**CFG5)
+    gen = torch.Generator().manual_seed(SEED)
+    params = OrderedDict()
+    for name, shape in ol.param_shapes(cfg).items():
+        params[name] = torch.randn(shape, generator=gen) * 0.02 if len(shape) >= 2 else torch.ones(shape)
+    ids = torch.randint(0, cfg.vocab_size, (8, 2049), generator=gen)
+    return cfg, params, ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
+
+
+def test_cfg5_llama50m_bf16_train_step(dev):
+    cfg, params, input_ids, labels = cfg5_inputs()
+    assert sum(p.numel() for p in params.values()) == 58_073_600
+    input_ids, labels = input_ids.to(dev), labels.to(dev)
+    # product path
+    model = LlamaForCausalLM(LlamaConfig(**CFG5)).to(dev)
+    load_into(model, params)
+    model = model.to(torch.bfloat16)
+    opt = MasterWeightsOptimizer(model.parameters(),
+                                 optimizer_factory=lambda ps: FusedAdamW(ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1))
+    before = [p.detach().clone() for p in model.parameters()]
+    loss = model({"input_ids": input_ids, "labels": labels})
+    loss.backward()
+    grad_norm = clip_grad_norm_(opt, 1.0)  # norm of the flat fp32 master grads, clip at 1.0
+    opt.step()
+    opt.zero_grad(set_to_none=True)
+    # oracle: (a) fp32 evaluation of the bf16-rounded network, (b) the reference-style eager bf16 evaluation
+    results = {}
+    for tag, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        leaves = OrderedDict((n, p.to(dev).to(torch.bfloat16).to(dtype).requires_grad_(True)) for n, p in params.items())
+        logits = ol.forward(leaves, cfg, input_ids)
+        ref_loss = F.cross_entropy(logits.float().view(-1, cfg.vocab_size), labels.view(-1))
+        ref_loss.backward()
+        results[tag] = (ref_loss.item(), oo.global_grad_norm([p.grad for p in leaves.values()]))
+        del logits, leaves
+    want_loss, want_norm = results["fp32"]
+    print(f"cfg5 loss hip={loss.item():.6f} fp32={want_loss:.6f} bf16-eager={results['bf16'][0]:.6f}; "
+          f"grad-norm hip={grad_norm:.6f} fp32={want_norm:.6f} bf16-eager={results['bf16'][1]:.6f}")
+    assert abs(loss.item() - want_loss) <= 1e-3 * want_loss
+    assert abs(grad_norm - want_norm) <= 1e-3 * want_norm
+    assert abs(results["bf16"][0] - want_loss) <= 2e-3 * want_loss  # the eager bf16 path itself is this close
+    # the step happened: every parameter moved by at most lr * (1 + wd |p|) and most moved
+    moved = 0
+    for p, b in zip(model.parameters(), before):
+        delta = (p.detach().float() - b.float()).abs()
+        assert delta.max() <= 3e-4 * 1.2 + 2.0 ** -8 * b.float().abs().max()
+        moved += int((delta > 0).sum())
+    assert moved > 0
+    for mp, p in zip(opt.master_params, model.parameters()):
+        assert torch.equal(p.detach(), mp.detach().to(torch.bfloat16))
