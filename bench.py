@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X hot path on ONE GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the headline workload over one synthetic batch: bf16 causal self-attention forward
+AND backward at B=4, H=16, S=4096, D=128 (the second benchmark configuration), inputs resident in HBM before
+the timed region.  `value` is the attention TFLOP/s over that step with the FlashAttention flop convention
+(forward 4*B*H*S^2*D/2, backward 2.5x forward).  The same JSON line also carries, under "extra", the other
+figures the metric names: fused AdamW GB/s on the LLaMA-50M flat buffers and LLaMA-50M train-step tokens/s.
+
+"roofline" describes the dominant kernel of the step (the one with the largest summed kernel time, measured
+live with HIP events on the launch stream through the library's timing hooks); "cpu_baseline" times the CPU
+oracle on a bounded sample of the same workload on the host cores.  Prints exactly one JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-extra", action="store_true", help="only the headline attention workload")
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    return ap.parse_args()
+
+
+def attention_inputs(torch, dev, B, H, S, D, seed=1234):
+    gen = torch.Generator().manual_seed(seed)
+    return [torch.randn(B, H, S, D, generator=gen).bfloat16().to(dev) for _ in range(4)]
+
+
+def timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_attention(torch, ops, _lib, dev, steps, warmup):
+    B, H, S, D = 4, 16, 4096, 128
+    q, k, v, do = attention_inputs(torch, dev, B, H, S, D)
+    fwd_flops = 4.0 * B * H * S * S * D / 2.0
+    flops = {"fwd": fwd_flops, "bwd": 2.5 * fwd_flops}
+    state = {}
+
+    def step():
+        o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_CAUSAL)
+        state["grads"] = ops.attention_backward(do, q, k, v, o, lse, mask_mode=ops.MASK_CAUSAL)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.kernel_timing(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    kernels = {}
+    for name in ("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"):
+        total_ms, launches = _lib.kernel_time_ms(name)
+        if launches:
+            kernels[name] = {"ms": total_ms / launches, "launches_per_step": launches / steps}
+    _lib.kernel_timing(False)
+    # algorithmic flops per launch of each kernel (FlashAttention convention: 2 GEMMs forward, 5 backward)
+    kernel_flops = {"attn_fwd": fwd_flops}
+    if "attn_bwd_dq" in kernels:  # split backward: dK/dV kernel carries 4 of the 5 GEMM-equivalents' share
+        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops * 0.6
+        kernel_flops["attn_bwd_dq"] = 2.5 * fwd_flops * 0.4
+    else:
+        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops
+    for name, rec in kernels.items():
+        rec["tflops"] = kernel_flops[name] / (rec["ms"] * 1e-3) / 1e12
+    return sec, flops, kernels, kernel_flops
+
+
+def bench_adamw(torch, ops, _lib, dev, steps, warmup):
+    n = 58_073_600  # LLaMA-50M parameters
+    p = torch.randn(n, device=dev)
+    g = torch.randn(n, device=dev) * 0.01
+    m = torch.zeros(n, device=dev)
+    v = torch.zeros(n, device=dev)
+    lowp = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    hp = dict(lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+    state = {"t": 0}
+
+    def step():
+        state["t"] += 1
+        ops.adamw_step_(p, g, m, v, step=state["t"], p_lowp=lowp, **hp)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.kernel_timing(True)
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    total_ms, launches = _lib.kernel_time_ms("adamw")
+    _lib.kernel_timing(False)
+    ms = total_ms / max(1, launches)
+    bytes_per_launch = 30.0 * n  # read p,g,m,v (16 B) + write p,m,v (12 B) + bf16 model copy (2 B)
+    return {"params": n, "bytes_per_param": 30, "kernel_ms": ms, "gbps": bytes_per_launch / (ms * 1e-3) / 1e9,
+            "frac_of_hbm_peak": bytes_per_launch / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+
+def bench_llama50m(torch, dev, steps, warmup):
+    from maltos_amd.grad_clip import clip_grad_norm_fused_
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+    from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
+
+    cfg = LlamaConfig(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8,
+                      num_attention_heads=8, max_position_embeddings=2048, rms_norm_eps=1e-5)
+    torch.manual_seed(1234)
+    model = LlamaForCausalLM(cfg)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() >= 2:
+                p.normal_(0.0, 0.02)
+    model = model.to(dev).to(torch.bfloat16)
+    opt = MasterWeightsOptimizer(model.parameters(), optimizer_factory=lambda ps: FusedAdamW(
+        ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1))
+    gen = torch.Generator().manual_seed(1234)
+    ids = torch.randint(0, cfg.vocab_size, (8, 2049), generator=gen).to(dev)
+    batch = {"input_ids": ids[:, :-1].contiguous(), "labels": ids[:, 1:].contiguous()}
+    out = {}
+
+    def step():
+        loss = model(batch)
+        loss.backward()
+        out["sq"] = clip_grad_norm_fused_(opt, 1.0)  # flat fp32 grads, global-norm clip at 1.0, no host sync
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        out["loss"] = loss
+
+    sec = timed(torch, step, steps, warmup)
+    tokens = 8 * 2048
+    return {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"]),
+            "grad_norm_last": float(out["sq"].sqrt()), "params": sum(p.numel() for p in model.parameters()),
+            "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12}
+
+
+def cpu_baseline(torch):
+    """CPU oracle (plain PyTorch fp32 restatement) on a bounded sample of the headline workload."""
+    from oracle import attention as oa
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    B, H, S, D = 1, 2, 4096, 128  # 1/32 of the B=4, H=16 workload, same S and D
+    gen = torch.Generator().manual_seed(1234)
+    q, k, v, do = (torch.randn(B, H, S, D, generator=gen).bfloat16().float() for _ in range(4))
+    mask = oa.causal_mask(S, S, "cpu")
+    flops = 3.5 * 4.0 * B * H * S * S * D / 2.0
+
+    def step():
+        qf, kf, vf = (t.clone().requires_grad_(True) for t in (q, k, v))
+        o, _ = oa.attention_with_lse(qf, kf, vf, mask)
+        o.backward(do)
+
+    step()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t0 < 10.0 and reps < 20):
+        step()
+        reps += 1
+    sec = (time.perf_counter() - t0) / reps
+    return {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle.attention (fp32 PyTorch restatement) fwd+bwd on B={B},H={H},S={S},D={D} "
+                      f"(1/32 of the workload, same S and D), {reps} repeats, {sec * 1e3:.0f} ms each"}
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}); every figure here is a single-GPU figure.",
+              file=sys.stderr)
+        return 2
+    import torch
+
+    from maltos_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the HIP path has no CPU fallback.", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    sec, flops, kernels, kernel_flops = bench_attention(torch, ops, _lib, dev, args.steps, args.warmup)
+    total_flops = flops["fwd"] + flops["bwd"]
+    value = total_flops / sec / 1e12
+    dominant = max(kernels, key=lambda n: kernels[n]["ms"] * kernels[n]["launches_per_step"])
+    dom = kernels[dominant]
+    result = {
+        "metric": "attn fwd+bwd TFLOP/s (% MFMA peak) S=4096; train tokens/sec LLaMA-50M, 1 GPU",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "causal self-attention fwd+bwd, B=4 H=16 S=4096 D=128, bf16 (configuration 2)",
+                   "flops_per_step": total_flops, "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS},
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": dom["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": dom["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "kernel_ms": dom["ms"], "algorithmic_flops_per_launch": kernel_flops[dominant]},
+        "kernels": kernels,
+    }
+    if not args.skip_extra:
+        extra = {}
+        extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
+        extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(2, args.warmup // 2))
+        result["extra"] = extra
+    if not args.skip_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

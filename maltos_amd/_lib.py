@@ -62,6 +62,8 @@ _SHAPE_P = C.POINTER(AttnShape)
 SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_abi_version": (C.c_int, []),
     "mlts_last_error": (C.c_char_p, []),
+    "mlts_kernel_timing_enable": (None, [C.c_int]),
+    "mlts_kernel_timing_read": (C.c_int, [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     "mlts_attn_supports": (C.c_char_p, [_SHAPE_P]),
     "mlts_attn_fwd_workspace_bytes": (C.c_int64, [_SHAPE_P]),
     "mlts_attn_bwd_workspace_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
@@ -139,6 +141,17 @@ def check(status: int) -> None:
     if status == MLTS_ERR_UNSUPPORTED:
         raise RuntimeError(msg)
     raise MaltosHipError(msg or f"libmaltos_hip status {status}")
+
+
+def kernel_timing(enable: bool) -> None:
+    lib().mlts_kernel_timing_enable(int(enable))
+
+
+def kernel_time_ms(name: str) -> tuple[float, int]:
+    """(summed kernel milliseconds, launches) recorded for `name` since timing was enabled."""
+    total, count = C.c_double(0.0), C.c_int64(0)
+    check(lib().mlts_kernel_timing_read(name.encode(), C.byref(total), C.byref(count)))
+    return total.value, count.value
 
 
 def strides3(values) -> C.Array:

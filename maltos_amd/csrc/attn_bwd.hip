@@ -449,7 +449,10 @@ int launch_bwd(const AttnBwdParams& bp, hipStream_t st) {
     configured = true;
   }
   const int64_t blocks = static_cast<int64_t>(bp.nkt) * bp.a.B * bp.a.Hkv;
-  if (blocks > 0) hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), smem, st, bp);
+  if (blocks > 0) {
+    MltsKernelTimer timer("attn_bwd_dkdv", st);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), smem, st, bp);
+  }
   return mlts_check_launch("mlts_attn_bwd");
 }
 

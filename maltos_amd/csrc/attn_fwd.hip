@@ -406,7 +406,10 @@ int launch_fwd(const AttnParams& p, hipStream_t st) {
     configured = true;
   }
   const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * p.Hq;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), smem, st, p);
+  {
+    MltsKernelTimer timer("attn_fwd", st);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), smem, st, p);
+  }
   return mlts_check_launch("mlts_attn_fwd");
 }
 

@@ -23,6 +23,17 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 void mlts_set_error(const char* fmt, ...);
 int mlts_check_launch(const char* what);
 
+// Optional per-kernel timing (mlts_kernel_timing_enable): brackets a launch with HIP events on the
+// launch stream.  Disabled by default; then the constructor and destructor are a single branch.
+struct MltsKernelTimer {
+  MltsKernelTimer(const char* name, hipStream_t stream);
+  ~MltsKernelTimer();
+  const char* name_;
+  hipStream_t stream_;
+  hipEvent_t start_;
+  bool active_;
+};
+
 #define MLTS_REQUIRE(cond, ...)        \
   do {                                 \
     if (!(cond)) {                     \

@@ -277,6 +277,7 @@ template <typename T>
 int rmsnorm_fwd_t(const void* x, const void* w, void* y, float* rstd, int64_t rows, int hidden, float eps,
                   hipStream_t st) {
   const int64_t blocks = (rows + kWaves - 1) / kWaves;
+  MltsKernelTimer timer("rmsnorm_fwd", st);
   hipLaunchKernelGGL(rmsnorm_fwd_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
                      static_cast<const T*>(w), static_cast<T*>(y), rstd, rows, hidden, eps);
   return mlts_check_launch("mlts_rmsnorm_fwd");
@@ -288,6 +289,7 @@ int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rst
   const int blocks = rmsnorm_bwd_blocks(rows);
   const int rows_per_block = static_cast<int>((rows + blocks - 1) / blocks);
   const size_t smem = static_cast<size_t>(kWaves) * hidden * sizeof(float);
+  MltsKernelTimer timer("rmsnorm_bwd", st);
   hipLaunchKernelGGL(rmsnorm_bwd_kernel<T>, dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy),
                      static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,
                      hidden, rows_per_block);

@@ -221,6 +221,7 @@ extern "C" int mlts_ce_fwd_bwd(const void* logits, const int64_t* labels, void* 
   float* row_loss = static_cast<float*>(workspace);
   hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, rows, ignore_index, count_out);
   if (rows > 0) {
+    MltsKernelTimer timer("ce", st);
     int rc = dtype == MLTS_BF16
                  ? ce_launch<bf16_t>(logits, labels, dlogits, row_loss, count_out, rows, vocab, ignore_index, st)
                  : ce_launch<float>(logits, labels, dlogits, row_loss, count_out, rows, vocab, ignore_index, st);

@@ -238,6 +238,7 @@ extern "C" int mlts_adamw_step(float* p, const float* g, float* m, float* v, voi
   const bool vec_ok = mlts_aligned16(p) && mlts_aligned16(g) && mlts_aligned16(m) && mlts_aligned16(v) &&
                       (plow == nullptr || (reinterpret_cast<uintptr_t>(plow) & 7u) == 0);
   int64_t done = 0;
+  MltsKernelTimer timer("adamw", st);
   if (vec_ok && n >= 4) {
     const int64_t nvec = n >> 2;
     const int64_t per_block = static_cast<int64_t>(kThreads) * kUnroll;
@@ -332,6 +333,7 @@ extern "C" int mlts_grad_to_f32(float* dst, const void* src, int32_t src_dtype, 
   hipStream_t st = static_cast<hipStream_t>(stream);
   double* partial = static_cast<double*>(workspace);
   int blocks;
+  MltsKernelTimer timer("grad_to_f32", st);
   if (src_dtype == MLTS_BF16 && mlts_aligned16(dst) && mlts_aligned16(src) && (n & 7) == 0 && n > 0) {
     blocks = grid_for(n >> 3, kSqBlocks);
     launch_grad_bf16_vec(acc, sq, blocks, st, dst, static_cast<const bf16_t*>(src), n >> 3, partial);
