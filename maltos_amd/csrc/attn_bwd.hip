@@ -1,20 +1,18 @@
-// Attention backward for gfx950 (bf16, head_dim 64/128): dQ, dK, dV by recompute from
-// (Q, K, V, O, LSE, dO) with v_mfma_f32_32x32x16_bf16.
+// Attention backward for gfx950 (bf16, head_dim 64/128), part 1 of 2: dK and dV by recompute from
+// (Q, K, V, LSE, delta, dO) with v_mfma_f32_32x32x16_bf16.  (dQ is part 2, attn_bwd_dq.hip; splitting the
+// backward pass costs two extra GEMMs of recompute but needs no atomics and no dS round trip.)
 //
 // A workgroup (4 wavefronts) owns 128 keys of one (batch, kv head) and walks the 64-row query
 // tiles that can see them, for every query head of the GQA group, so dK/dV are accumulated in
-// registers and written exactly once (no atomics, native GQA).  Per tile and wavefront (32 keys):
+// registers and written exactly once (native GQA, deterministic).  Per tile and wavefront (32 keys):
 //     S  = Q K^T        A = Q  (LDS, row major)      B = K  (registers, loaded once)
 //     dP = dO V^T       A = dO (LDS, row major)      B = V  (registers, loaded once)
 //     P  = exp2(S c - LSE), dS = P (dP - delta)       in registers, lane = key, in-lane = query
 //     dV += P^T dO      A = P^T  (registers as is)   B = dO^T (LDS, transposed while staging)
 //     dK += dS^T Q      A = dS^T (registers as is)   B = Q^T  (LDS, transposed while staging)
-//     dQ^T = K^T dS^T   A = K^T (registers, once)    B = dS^T from LDS after one 2-byte scatter
-// The accumulator layout of S is the A-operand layout of the dV/dK products, so only dS makes a
-// round trip through LDS, for dQ.  dQ partial sums (one per key tile) go to an fp32 buffer with
-// hardware float atomics and are converted once at the end.
+// The accumulator layout of S is the A-operand layout of the dV/dK products, so P and dS never leave
+// registers.  Q/dO tiles are double buffered in LDS: one barrier per tile.
 #include "attn_common.hpp"
-#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 namespace {
 
@@ -22,21 +20,19 @@ constexpr int BKV = 128;
 constexpr int BQ = 64;
 constexpr int WAVES = 4;
 constexpr int THREADS = 256;
-constexpr int DS_STR = BKV + 8;
 
 template <int D>
 struct BwdLds {
   static constexpr int RSTR = D + 8;
   static constexpr int ROW_ELEMS = BQ * RSTR;     // row-major tile
   static constexpr int T_ELEMS = D * BQ;          // transposed tile
-  static constexpr int DS_ELEMS = BQ * DS_STR;    // one dS buffer
   static constexpr int OFF_Q = 0;
   static constexpr int OFF_DO = OFF_Q + ROW_ELEMS;
   static constexpr int OFF_QT = OFF_DO + ROW_ELEMS;
   static constexpr int OFF_DOT = OFF_QT + T_ELEMS;
-  static constexpr int OFF_DS = OFF_DOT + T_ELEMS;
-  static constexpr int OFF_STAT = OFF_DS + DS_ELEMS;  // lse[64], delta[64] as floats
-  static constexpr int BYTES = OFF_STAT * 2 + 2 * BQ * 4;
+  static constexpr int OFF_STAT = OFF_DOT + T_ELEMS;  // lse[64], delta[64] as floats
+  static constexpr int STAGE = OFF_STAT + 4 * BQ;     // in bf16 elements (the two float arrays take 4 * BQ)
+  static constexpr int BYTES = 2 * STAGE * 2;
 };
 
 __device__ __forceinline__ int t_swz(int d) { return ((d >> 1) ^ (d >> 3)) & 7; }
@@ -53,17 +49,9 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
   constexpr int DB = D / 32;
   constexpr int VEC = D / 16;        // elements per thread per staged row
   constexpr int VW = VEC / 2;        // dwords
-  constexpr int DQ_QB = D == 128 ? 2 : 1;  // query blocks of the dQ product per wavefront
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* smem = reinterpret_cast<bf16_t*>(smem_raw);
-  bf16_t* sQ = smem + L::OFF_Q;
-  bf16_t* sdO = smem + L::OFF_DO;
-  uint16_t* sQt = reinterpret_cast<uint16_t*>(smem + L::OFF_QT);
-  uint16_t* sdOt = reinterpret_cast<uint16_t*>(smem + L::OFF_DOT);
-  bf16_t* sdS = smem + L::OFF_DS;
-  float* sLse = reinterpret_cast<float*>(smem + L::OFF_STAT);
-  float* sDelta = sLse + BQ;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
@@ -80,7 +68,7 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
 
-  // ---- K, V fragments (B operands) and K^T fragments (A operand of the dQ product) --------
+  // ---- K, V fragments (B operands), loaded once -----------------------------------------
   bf16x8 kf[KS], vf[KS];
   {
     const int row = wkv0 + l32;
@@ -98,21 +86,6 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
       }
     }
   }
-  const int dq_db = D == 128 ? wave : (wave & 1);
-  const int dq_qb0 = D == 128 ? 0 : (wave >> 1);
-  bf16x8 ktf[BKV / 16];
-  {
-    const int d = dq_db * 32 + l32;
-#pragma unroll
-    for (int t = 0; t < BKV / 16; ++t) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = kv0 + t * 16 + hh * 8 + i;
-        ktf[t][i] = row < p.Sk ? K[static_cast<int64_t>(row) * p.ks[2] + d] : static_cast<bf16_t>(0.f);
-      }
-    }
-  }
-
   // ---- query-tile range -------------------------------------------------------------------
   const int nqt = (p.Sq + BQ - 1) / BQ;
   int qt_begin = 0;
@@ -201,7 +174,14 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
     }
   };
 
-  auto lds_store = [&]() {
+  auto lds_store = [&](int stage) {
+    bf16_t* base = smem + stage * L::STAGE;
+    bf16_t* sQ = base + L::OFF_Q;
+    bf16_t* sdO = base + L::OFF_DO;
+    uint16_t* sQt = reinterpret_cast<uint16_t*>(base + L::OFF_QT);
+    uint16_t* sdOt = reinterpret_cast<uint16_t*>(base + L::OFF_DOT);
+    float* sLse = reinterpret_cast<float*>(base + L::OFF_STAT);
+    float* sDelta = sLse + BQ;
     const int slot0 = t_slot(s_grp * 4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -258,12 +238,19 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
 
   int it = next_it(0);
   if (it < total_it) gload(it);
+  int stage = 0;
   while (it < total_it) {
-    const int hq = hkv * group + it / span;
     const int qt = qt_begin + it % span;
     const int q0 = qt * BQ;
-    lds_store();
+    lds_store(stage);
     __syncthreads();
+    const bf16_t* base = smem + stage * L::STAGE;
+    const bf16_t* sQ = base + L::OFF_Q;
+    const bf16_t* sdO = base + L::OFF_DO;
+    const uint16_t* sQt = reinterpret_cast<const uint16_t*>(base + L::OFF_QT);
+    const uint16_t* sdOt = reinterpret_cast<const uint16_t*>(base + L::OFF_DOT);
+    const float* sLse = reinterpret_cast<const float*>(base + L::OFF_STAT);
+    const float* sDelta = sLse + BQ;
     const int itn = next_it(it + 1);
     if (itn < total_it) gload(itn);
 
@@ -278,7 +265,6 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
     if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || q0 + BQ > p.Sq)) cls = TILE_MASKED;
     if (wkv0 >= p.Sk) cls = TILE_SKIP;
 
-    bf16_t* dsb = sdS;  // rewritten only after the barrier that follows the next tile's staging
     if (cls != TILE_SKIP) {
       // P and dS in registers; lane = key (wkv0 + l32), register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4
       bf16x8 pfr[2][2], dsfr[2][2];
@@ -328,7 +314,6 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
             const float dsv = pv * (dpacc[e] - dl4[r]);
             pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
             dsfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(dsv);
-            dsb[(qrow + r) * DS_STR + wave * 32 + l32] = static_cast<bf16_t>(dsv);
           }
         }
       }
@@ -346,41 +331,9 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
           dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsfr[c >> 1][c & 1], qb_, dkacc[db], 0, 0, 0);
         }
       }
-    } else {
-      // this wavefront's keys see none of the tile: its slice of dS is zero
-#pragma unroll
-      for (int i = 0; i < BQ / 2; ++i) dsb[(i * 2 + hh) * DS_STR + wave * 32 + l32] = static_cast<bf16_t>(0.f);
-    }
-    __syncthreads();
-
-    // ---- dQ^T block of this wavefront over all 128 keys ----
-    {
-      f32x16 dqacc[DQ_QB];
-#pragma unroll
-      for (int qi = 0; qi < DQ_QB; ++qi)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) dqacc[qi][e] = 0.f;
-#pragma unroll
-      for (int t = 0; t < BKV / 16; ++t) {
-#pragma unroll
-        for (int qi = 0; qi < DQ_QB; ++qi) {
-          const int qb = dq_qb0 + qi;
-          const bf16x8 dsB = *reinterpret_cast<const bf16x8*>(dsb + (qb * 32 + l32) * DS_STR + t * 16 + hh * 8);
-          dqacc[qi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[t], dsB, dqacc[qi], 0, 0, 0);
-        }
-      }
-      float* dqh = bp.dq_acc + b * bp.dqs[0] + hq * bp.dqs[1];
-#pragma unroll
-      for (int qi = 0; qi < DQ_QB; ++qi) {
-        const int row = q0 + (dq_qb0 + qi) * 32 + l32;
-        if (row < p.Sq) {
-          float* dst = dqh + static_cast<int64_t>(row) * bp.dqs[2] + dq_db * 32 + hh * 4;
-#pragma unroll
-          for (int e = 0; e < 16; ++e) unsafeAtomicAdd(dst + (e >> 2) * 8 + (e & 3), dqacc[qi][e] * p.scale);
-        }
-      }
     }
     it = itn;
+    stage ^= 1;
   }
 
   // ---- write dK, dV: register e <-> key wkv0 + 8 (e/4) + 4 hh + e%4, lane -> head-dim column ----
@@ -405,36 +358,6 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
   }
 }
 
-__global__ __launch_bounds__(256) void zero_f32_kernel(float* x, int64_t nvec) {
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
-  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < nvec; i += stride)
-    reinterpret_cast<f32x4*>(x)[i] = z;
-}
-
-// dq[b, h, s, :] (bf16, strided) = bf16(acc[b, h, s, :]) ; acc contiguous fp32
-__global__ __launch_bounds__(256) void dq_convert_kernel(const float* __restrict__ acc, bf16_t* __restrict__ dq,
-                                                         int64_t s0, int64_t s1, int64_t s2, int H, int S, int D,
-                                                         int64_t total_vec) {
-  const int vpr = D / 8;
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (idx >= total_vec) return;
-  const int vc = static_cast<int>(idx % vpr);
-  const int64_t row = idx / vpr;
-  const int s = static_cast<int>(row % S);
-  const int h = static_cast<int>((row / S) % H);
-  const int b = static_cast<int>(row / (static_cast<int64_t>(S) * H));
-  const f32x4 a = reinterpret_cast<const f32x4*>(acc + row * D)[vc * 2];
-  const f32x4 c = reinterpret_cast<const f32x4*>(acc + row * D)[vc * 2 + 1];
-  bf16x8 o;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    o[e] = static_cast<bf16_t>(a[e]);
-    o[4 + e] = static_cast<bf16_t>(c[e]);
-  }
-  *reinterpret_cast<bf16x8*>(dq + b * s0 + h * s1 + static_cast<int64_t>(s) * s2 + vc * 8) = o;
-}
-
 template <int D, int MODE>
 int launch_bwd(const AttnBwdParams& bp, hipStream_t st) {
   auto kern = attn_bwd_kernel<D, MODE>;
@@ -456,33 +379,20 @@ int launch_bwd(const AttnBwdParams& bp, hipStream_t st) {
   return mlts_check_launch("mlts_attn_bwd");
 }
 
-inline int64_t align256(int64_t x) { return (x + 255) & ~255LL; }
-
 }  // namespace
 
+int mlts_attn_bwd_dq_bf16(const AttnBwdParams& bp, int D, int mode, hipStream_t st);
+
 int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32) {
-  if (accumulate_f32) return 0;
-  return align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * s->D * 4);
+  (void)s;
+  (void)accumulate_f32;
+  return 0;
 }
 
 int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
+  (void)workspace;
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
-  bf16_t* dq_out = reinterpret_cast<bf16_t*>(bp.dq_acc);
-  int64_t dq_out_stride[3] = {bp.dqs[0], bp.dqs[1], bp.dqs[2]};
-  const int64_t n = static_cast<int64_t>(p.B) * p.Hq * p.Sq * D;
-  if (!bp.accumulate_f32) {
-    float* acc = static_cast<float*>(workspace);
-    if (n > 0) {
-      int64_t blocks = (n / 4 + 255) / 256;
-      if (blocks > 65536) blocks = 65536;
-      hipLaunchKernelGGL(zero_f32_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, acc, n / 4);
-    }
-    bp.dq_acc = acc;
-    bp.dqs[0] = static_cast<int64_t>(p.Hq) * p.Sq * D;
-    bp.dqs[1] = static_cast<int64_t>(p.Sq) * D;
-    bp.dqs[2] = D;
-  }
   int rc;
   if (D == 128) {
     if (mode == MLTS_MASK_NONE) rc = launch_bwd<128, MLTS_MASK_NONE>(bp, st);
@@ -494,11 +404,5 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
-  if (!bp.accumulate_f32 && n > 0) {
-    const int64_t total_vec = n / 8;
-    hipLaunchKernelGGL(dq_convert_kernel, dim3(static_cast<unsigned>((total_vec + 255) / 256)), dim3(256), 0, st,
-                       bp.dq_acc, dq_out, dq_out_stride[0], dq_out_stride[1], dq_out_stride[2], p.Hq, p.Sq, D, total_vec);
-    return mlts_check_launch("mlts_attn_bwd");
-  }
-  return MLTS_OK;
+  return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

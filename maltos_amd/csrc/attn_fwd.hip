@@ -16,14 +16,11 @@
 //     (min/max position, min/max sequence id) statistics to skip or fast-path whole tiles and fall
 //     back to the element predicate only on tiles that straddle a boundary.
 #include "attn_common.hpp"
+#include <stdlib.h>
 
 namespace {
 
 constexpr int BN = 64;          // keys per tile
-constexpr int WAVES = 4;
-constexpr int THREADS = WAVES * 64;
-constexpr int QB = 2;           // 32-row query blocks per wavefront
-constexpr int BM = WAVES * QB * 32;
 
 template <int D>
 struct FwdLds {
@@ -46,14 +43,22 @@ __device__ __forceinline__ int vt_slot(int r) {
   return (((kb * 2 + t) * 2 + hh) << 3) + (ihi << 2) + (r & 3);
 }
 
-template <int D, int MODE>
-__global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p) {
+// WAVES x QB: 4 x 2 (one wavefront per SIMD, 64 query rows each, up to 512 registers) or
+// 8 x 1 (two wavefronts per SIMD, 32 query rows each, <= 256 registers: the hardware overlaps one
+// wavefront's softmax VALU work with the other's MFMAs).  Both cover 256 query rows per workgroup.
+template <int D, int MODE, int WAVES, int QB>
+__global__ __launch_bounds__(WAVES * 64) void attn_fwd_kernel(const AttnParams p) {
   using L = FwdLds<D>;
+  constexpr int THREADS = WAVES * 64;
+  constexpr int BM = WAVES * QB * 32;
+  constexpr int WROWS = QB * 32;     // query rows per wavefront
   constexpr int KS = D / 16;    // k-steps of the score product
   constexpr int DB = D / 32;    // 32-row blocks of O^T
-  constexpr int KLD = D / 32;   // 16-byte K vectors staged per thread
+  constexpr int KLD = D / 32;   // 16-byte K vectors staged per thread (256 staging threads)
   constexpr int TPR = D / 8;    // threads per K row
-  constexpr int VEC = D / 16;   // V elements per thread per row (4 rows per thread)
+  constexpr int VEC = D / 16;   // V elements per thread per row (4 rows per thread, 256 staging threads)
+  // with 8 wavefronts, threads 0..255 stage V (transposing) and threads 256..511 stage K
+  constexpr bool SPLIT = WAVES == 8;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* smem = reinterpret_cast<bf16_t*>(smem_raw);
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
   const int b = bh / p.Hq, hq = bh % p.Hq;
   const int hkv = hq / (p.Hq / p.Hkv);
   const int q0 = qt * BM;
-  const int wq0 = q0 + wave * 64;
+  const int wq0 = q0 + wave * WROWS;
 
   const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
   // per-lane query metadata for the document mask
   int qpos[QB], qseq[QB];
   int4 wq_stats = make_int4(0, -1, 0, -1);
-  int4 bq_stats[WAVES];
+  int4 bq_stats[BM / 64];
   if (MODE == MLTS_MASK_DOC) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -104,12 +109,12 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
       qseq[qb] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + row] : -1;
     }
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
+    for (int w = 0; w < BM / 64; ++w) {
       const int t = (q0 >> 6) + w;
       bq_stats[w] = t < p.nq_stats ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
     }
     {
-      const int t = (q0 >> 6) + wave;
+      const int t = wq0 >> 6;  // statistics are per 64 query rows; a 32-row wavefront uses its parent's
       if (t < p.nq_stats) wq_stats = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t];
     }
   }
@@ -122,14 +127,14 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
     const int lim = last_q + p.causal_off;  // last visible key index for the block
     j_end = lim < 0 ? 0 : min(nkt, lim / BN + 1);
   }
-  const int wave_last_q = min(wq0 + 63, p.Sq - 1);
+  const int wave_last_q = min(wq0 + WROWS - 1, p.Sq - 1);
 
   auto block_needs = [&](int j) -> bool {
     if (MODE != MLTS_MASK_DOC) return true;
     const int4 ks4 = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
     bool need = false;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
+    for (int w = 0; w < BM / 64; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
     return need;
   };
   auto next_tile = [&](int j) -> int {
@@ -140,14 +145,17 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
   // ---- staging registers and helpers ------------------------------------------------------
   bf16x8 kreg[KLD];
   uint16_t vreg[4][VEC];
-  const int k_row0 = tid / TPR, k_col = (tid % TPR) * 8;
-  const int v_grp = tid >> 4, v_d0 = (tid & 15) * VEC;
+  const int stid = tid & 255;  // index among the 256 threads that share a staging role
+  const bool do_k = !SPLIT || tid >= 256, do_v = !SPLIT || tid < 256;
+  const int k_row0 = stid / TPR, k_col = (stid % TPR) * 8;
+  const int v_grp = stid >> 4, v_d0 = (stid & 15) * VEC;
 
   auto gload = [&](int j) {
     const int kv0 = j * BN;
+    if (do_k) {
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
-      const int r = kv0 + k_row0 + i * (THREADS / TPR);
+      const int r = kv0 + k_row0 + i * (256 / TPR);
       if (r < p.Sk) {
         kreg[i] = *reinterpret_cast<const bf16x8*>(K + static_cast<int64_t>(r) * p.ks[2] + k_col);
       } else {
@@ -155,6 +163,8 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
         for (int e = 0; e < 8; ++e) kreg[i][e] = static_cast<bf16_t>(0.f);
       }
     }
+    }
+    if (do_v) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = kv0 + v_grp * 4 + i;
@@ -180,17 +190,21 @@ __global__ __launch_bounds__(THREADS, 1) void attn_fwd_kernel(const AttnParams p
         for (int e = 0; e < VEC; ++e) vreg[i][e] = 0;
       }
     }
+    }
   };
 
   auto lds_store = [&](int stage) {
     bf16_t* sK = smem + stage * L::STAGE;
     uint16_t* sV = reinterpret_cast<uint16_t*>(smem + stage * L::STAGE + L::K_ELEMS);
+    if (do_k) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) {
-      const int r = k_row0 + i * (THREADS / TPR);
-      *reinterpret_cast<bf16x8*>(sK + r * L::KSTR + k_col) = kreg[i];
+      for (int i = 0; i < KLD; ++i) {
+        const int r = k_row0 + i * (256 / TPR);
+        *reinterpret_cast<bf16x8*>(sK + r * L::KSTR + k_col) = kreg[i];
+      }
     }
     const int slot0 = vt_slot(v_grp * 4);  // 4 consecutive rows -> 4 consecutive slots
+    if (do_v)
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       const int d = v_d0 + e;
@@ -392,9 +406,10 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
   if (threadIdx.x == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
 }
 
-template <int D, int MODE>
+template <int D, int MODE, int WAVES, int QB>
 int launch_fwd(const AttnParams& p, hipStream_t st) {
-  auto kern = attn_fwd_kernel<D, MODE>;
+  constexpr int THREADS = WAVES * 64;
+  auto kern = attn_fwd_kernel<D, MODE, WAVES, QB>;
   constexpr int smem = FwdLds<D>::BYTES;
   static bool configured = false;  // per template instance; the attribute is sticky per function
   if (!configured && smem > 48 * 1024) {
@@ -421,14 +436,26 @@ void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S
   hipLaunchKernelGGL(tile_stats_kernel, dim3(B * ntiles), dim3(64), 0, st, pos, seq, S, ntiles, out);
 }
 
-int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st) {
-  p.nqt = (p.Sq + BM - 1) / BM;
+namespace {
+template <int WAVES, int QB>
+int dispatch_fwd(AttnParams p, int D, int mode, hipStream_t st) {
+  p.nqt = (p.Sq + WAVES * QB * 32 - 1) / (WAVES * QB * 32);
   if (D == 128) {
-    if (mode == MLTS_MASK_NONE) return launch_fwd<128, MLTS_MASK_NONE>(p, st);
-    if (mode == MLTS_MASK_CAUSAL) return launch_fwd<128, MLTS_MASK_CAUSAL>(p, st);
-    return launch_fwd<128, MLTS_MASK_DOC>(p, st);
+    if (mode == MLTS_MASK_NONE) return launch_fwd<128, MLTS_MASK_NONE, WAVES, QB>(p, st);
+    if (mode == MLTS_MASK_CAUSAL) return launch_fwd<128, MLTS_MASK_CAUSAL, WAVES, QB>(p, st);
+    return launch_fwd<128, MLTS_MASK_DOC, WAVES, QB>(p, st);
   }
-  if (mode == MLTS_MASK_NONE) return launch_fwd<64, MLTS_MASK_NONE>(p, st);
-  if (mode == MLTS_MASK_CAUSAL) return launch_fwd<64, MLTS_MASK_CAUSAL>(p, st);
-  return launch_fwd<64, MLTS_MASK_DOC>(p, st);
+  if (mode == MLTS_MASK_NONE) return launch_fwd<64, MLTS_MASK_NONE, WAVES, QB>(p, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch_fwd<64, MLTS_MASK_CAUSAL, WAVES, QB>(p, st);
+  return launch_fwd<64, MLTS_MASK_DOC, WAVES, QB>(p, st);
+}
+}  // namespace
+
+int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st) {
+  static const int variant = [] {
+    const char* e = getenv("MLTS_FWD_VARIANT");  // tuning aid: "4x2" selects the one-wavefront-per-SIMD form
+    return (e && e[0] == '4') ? 4 : 8;
+  }();
+  if (variant == 4) return dispatch_fwd<4, 2>(p, D, mode, st);
+  return dispatch_fwd<8, 1>(p, D, mode, st);
 }
