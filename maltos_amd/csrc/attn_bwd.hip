@@ -13,6 +13,7 @@
 // The accumulator layout of S is the A-operand layout of the dV/dK products, so P and dS never leave
 // registers.  Q/dO tiles are double buffered in LDS: one barrier per tile.
 #include "attn_common.hpp"
+#include <type_traits>
 
 namespace {
 
@@ -35,7 +36,7 @@ struct BwdLds {
   static constexpr int BYTES = 2 * STAGE * 2;
 };
 
-__device__ __forceinline__ int t_swz(int d) { return ((d >> 1) ^ (d >> 3)) & 7; }
+__device__ __forceinline__ int t_swz(int d) { return ((d >> 1) ^ (d >> 4)) & 7; }
 __device__ __forceinline__ int t_slot(int r) {
   const int kb = r >> 5, t = (r >> 4) & 1, grp = (r >> 2) & 3;
   return (((kb * 2 + t) * 2 + (grp & 1)) << 3) + ((grp >> 1) << 2) + (r & 3);
@@ -169,8 +170,13 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
     if (tid < 2 * BQ) {
       const int r = q0 + (tid & (BQ - 1));
       const int64_t off = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + r;
-      if (tid < BQ) stat_reg = r < p.Sq ? p.lse[off] : -INFINITY;
-      else stat_reg = r < p.Sq ? bp.delta[off] : 0.f;
+      if (tid < BQ) {
+        // stored as lse * log2(e); +inf for rows that saw no key (or lie beyond Sq) makes exp2(s - lse2) = 0
+        const float l = r < p.Sq ? p.lse[off] : -INFINITY;
+        stat_reg = l == -INFINITY ? INFINITY : l * kLog2e;
+      } else {
+        stat_reg = r < p.Sq ? bp.delta[off] : 0.f;
+      }
     }
   };
 
@@ -284,38 +290,42 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_kernel(const AttnBwdParam
           const bf16x8 da = *reinterpret_cast<const bf16x8*>(sdO + (qb * 32 + l32) * L::RSTR + ks * 16 + hh * 8);
           dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[ks], dpacc, 0, 0, 0);
         }
+        auto softmax_bwd = [&](auto masked_tag) {
+          constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int qrow = qb * 32 + g * 8 + hh * 4;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sLse + qrow);
-          const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDelta + qrow);
-          int qp4[4], qs4[4];
-          if (MODE == MLTS_MASK_DOC && cls == TILE_MASKED) {
+          for (int g = 0; g < 4; ++g) {
+            const int qrow = qb * 32 + g * 8 + hh * 4;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sLse + qrow);  // already lse * log2(e)
+            const f32x4 dl4 = *reinterpret_cast<const f32x4*>(sDelta + qrow);
+            int qp4[4], qs4[4];
+            if (MASKED && MODE == MLTS_MASK_DOC) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int qi = q0 + qrow + r;
+                const bool ok = qi < p.Sq;
+                qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
+                qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
+              }
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int qi = q0 + qrow + r;
-              const bool ok = qi < p.Sq;
-              qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
-              qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
+              const int e = g * 4 + r;
+              float pv = __builtin_amdgcn_exp2f(sacc[e] * p.scale_log2 - lse4[r]);
+              if (MASKED) {
+                const int qi = q0 + qrow + r;
+                bool vis = kj < p.Sk && qi < p.Sq;
+                if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qi + p.causal_off);
+                if (MODE == MLTS_MASK_DOC) vis = vis && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
+                if (!vis) pv = 0.f;
+              }
+              const float dsv = pv * (dpacc[e] - dl4[r]);
+              pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
+              dsfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(dsv);
             }
           }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int e = g * 4 + r;
-            const float lse2 = lse4[r] == -INFINITY ? INFINITY : lse4[r] * kLog2e;
-            float pv = __builtin_amdgcn_exp2f(sacc[e] * p.scale_log2 - lse2);
-            if (cls == TILE_MASKED) {
-              const int qi = q0 + qrow + r;
-              bool vis = kj < p.Sk && qi < p.Sq;
-              if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qi + p.causal_off);
-              if (MODE == MLTS_MASK_DOC) vis = vis && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
-              if (!vis) pv = 0.f;
-            }
-            const float dsv = pv * (dpacc[e] - dl4[r]);
-            pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
-            dsfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(dsv);
-          }
-        }
+        };
+        if (cls == TILE_MASKED) softmax_bwd(std::true_type{});
+        else softmax_bwd(std::false_type{});
       }
 
       // dV += P^T dO, dK += dS^T Q

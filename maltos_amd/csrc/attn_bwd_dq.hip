@@ -11,6 +11,7 @@
 // no atomics.  Two wavefronts per SIMD (<= 256 registers) let the hardware overlap one wavefront's
 // exp2/VALU work with the other's MFMAs.
 #include "attn_common.hpp"
+#include <type_traits>
 
 namespace {
 
@@ -31,7 +32,7 @@ struct DqLds {
   static constexpr int BYTES = 2 * STAGE * 2;
 };
 
-__device__ __forceinline__ int q_swz(int d) { return ((d >> 1) ^ (d >> 3)) & 7; }
+__device__ __forceinline__ int q_swz(int d) { return ((d >> 1) ^ (d >> 4)) & 7; }
 __device__ __forceinline__ int q_slot(int r) {
   const int kb = r >> 5, t = (r >> 4) & 1, grp = (r >> 2) & 3;
   return (((kb * 2 + t) * 2 + (grp & 1)) << 3) + ((grp >> 1) << 2) + (r & 3);
@@ -133,8 +134,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
   const bool do_k = tid < 256;
   const int s_grp = stid >> 4, s_d0 = (stid & 15) * VEC;
   const int v_row0 = stid / TPR, v_col = (stid % TPR) * 8;
-  uint32_t kreg[4][VW];
-  bf16x8 vreg[KLD];
+  uint32_t st[D / 8];  // one staging buffer for both roles: K rows [4][VW] words, or V vectors [KLD][4] words
 
   auto gload = [&](int j) {
     const int kv0 = j * BN;
@@ -147,27 +147,25 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
           if (VW == 4) {
             const u32x4 a = *reinterpret_cast<const u32x4*>(src);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) kreg[i][e] = a[e];
+            for (int e = 0; e < 4; ++e) st[i * VW + e] = a[e];
           } else {
             const u32x2 a = *reinterpret_cast<const u32x2*>(src);
 #pragma unroll
-            for (int e = 0; e < 2; ++e) kreg[i][e] = a[e];
+            for (int e = 0; e < 2; ++e) st[i * VW + e] = a[e];
           }
         } else {
 #pragma unroll
-          for (int e = 0; e < VW; ++e) kreg[i][e] = 0u;
+          for (int e = 0; e < VW; ++e) st[i * VW + e] = 0u;
         }
       }
     } else {
 #pragma unroll
       for (int i = 0; i < KLD; ++i) {
         const int r = kv0 + v_row0 + i * (256 / TPR);
-        if (r < p.Sk) {
-          vreg[i] = *reinterpret_cast<const bf16x8*>(V + static_cast<int64_t>(r) * p.vs[2] + v_col);
-        } else {
+        u32x4 a = {0u, 0u, 0u, 0u};
+        if (r < p.Sk) a = *reinterpret_cast<const u32x4*>(V + static_cast<int64_t>(r) * p.vs[2] + v_col);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) vreg[i][e] = static_cast<bf16_t>(0.f);
-        }
+        for (int e = 0; e < 4; ++e) st[i * 4 + e] = a[e];
       }
     }
   };
@@ -183,12 +181,12 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
         if (VW == 4) {
           u32x4 a;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) a[e] = kreg[i][e];
+          for (int e = 0; e < 4; ++e) a[e] = st[i * VW + e];
           *reinterpret_cast<u32x4*>(dst) = a;
         } else {
           u32x2 a;
 #pragma unroll
-          for (int e = 0; e < 2; ++e) a[e] = kreg[i][e];
+          for (int e = 0; e < 2; ++e) a[e] = st[i * VW + e];
           *reinterpret_cast<u32x2*>(dst) = a;
         }
       }
@@ -199,8 +197,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
         const int chunk = (slot0 >> 3) ^ q_swz(d);
         const int sh = (e & 1) * 16, w = e >> 1;
         u32x2 a;
-        a[0] = ((kreg[0][w] >> sh) & 0xffffu) | (((kreg[1][w] >> sh) & 0xffffu) << 16);
-        a[1] = ((kreg[2][w] >> sh) & 0xffffu) | (((kreg[3][w] >> sh) & 0xffffu) << 16);
+        a[0] = ((st[0 * VW + w] >> sh) & 0xffffu) | (((st[1 * VW + w] >> sh) & 0xffffu) << 16);
+        a[1] = ((st[2 * VW + w] >> sh) & 0xffffu) | (((st[3 * VW + w] >> sh) & 0xffffu) << 16);
         *reinterpret_cast<u32x2*>(sKt + d * BN + (chunk << 3) + (slot0 & 7)) = a;
       }
     } else {
@@ -208,7 +206,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
 #pragma unroll
       for (int i = 0; i < KLD; ++i) {
         const int r = v_row0 + i * (256 / TPR);
-        *reinterpret_cast<bf16x8*>(sV + r * L::RSTR + v_col) = vreg[i];
+        u32x4 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = st[i * 4 + e];
+        *reinterpret_cast<u32x4*>(sV + r * L::RSTR + v_col) = a;
       }
     }
   };
@@ -244,54 +245,55 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_kernel(const AttnBwdParam
       const bf16_t* sK = base + L::OFF_K;
       const bf16_t* sV = base + L::OFF_V;
       const bf16_t* sKt = base + L::OFF_KT;
-      f32x16 sacc[2], dpacc[2];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          sacc[kb][e] = 0.f;
-          dpacc[kb][e] = 0.f;
-        }
+      bf16x8 dsf[4];
+      // one 32-key block at a time keeps only one S and one dP accumulator live
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
+        f32x16 sacc, dpacc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          sacc[e] = 0.f;
+          dpacc[e] = 0.f;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8 ka = *reinterpret_cast<const bf16x8*>(sK + (kb * 32 + l32) * L::RSTR + ks * 16 + hh * 8);
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], sacc[kb], 0, 0, 0);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[ks], sacc, 0, 0, 0);
           const bf16x8 va = *reinterpret_cast<const bf16x8*>(sV + (kb * 32 + l32) * L::RSTR + ks * 16 + hh * 8);
-          dpacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[ks], dpacc[kb], 0, 0, 0);
+          dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[ks], dpacc, 0, 0, 0);
         }
-      }
-      bf16x8 dsf[4];
+        auto softmax_bwd = [&](auto masked_tag) {
+          constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+          for (int g = 0; g < 4; ++g) {
+            const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+            int kp[4], ksq[4];
+            if (MASKED && MODE == MLTS_MASK_DOC) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
-          int kp[4], ksq[4];
-          if (MODE == MLTS_MASK_DOC && cls == TILE_MASKED) {
+              for (int r = 0; r < 4; ++r) {
+                const int kj = kbase + r;
+                const bool ok = kj < p.Sk;
+                kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
+                ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
+              }
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const int kj = kbase + r;
-              const bool ok = kj < p.Sk;
-              kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
-              ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
+              const int e = g * 4 + r;
+              float pv = __builtin_amdgcn_exp2f(sacc[e] * p.scale_log2 - lse2);
+              if (MASKED) {
+                const int kj = kbase + r;
+                bool vis = kj < p.Sk;
+                if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
+                if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+                if (!vis) pv = 0.f;
+              }
+              dsf[kb * 2 + (e >> 3)][e & 7] = static_cast<bf16_t>(pv * (dpacc[e] - delta));
             }
           }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int e = g * 4 + r;
-            float pv = __builtin_amdgcn_exp2f(sacc[kb][e] * p.scale_log2 - lse2);
-            if (cls == TILE_MASKED) {
-              const int kj = kbase + r;
-              bool vis = kj < p.Sk;
-              if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
-              if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
-              if (!vis) pv = 0.f;
-            }
-            dsf[kb * 2 + (e >> 3)][e & 7] = static_cast<bf16_t>(pv * (dpacc[kb][e] - delta));
-          }
-        }
+        };
+        if (cls == TILE_MASKED) softmax_bwd(std::true_type{});
+        else softmax_bwd(std::false_type{});
       }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
