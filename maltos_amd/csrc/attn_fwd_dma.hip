@@ -1,0 +1,403 @@
+// Attention forward, head_dim 128, bf16: the gfx950 memory pipeline version.
+//
+// Same math and register layouts as attn_fwd.hip (S^T = K Q^T, P in registers, O^T = V^T P^T, eight
+// wavefronts x 32 query rows), but K and V tiles travel global -> LDS with the 16-byte LDS-DMA loads
+// (global_load_lds_dwordx4: no staging registers, no ds_write, no VALU work) into a three-stage ring, so a
+// tile's loads are issued two tiles ahead of its use.  Tiles are stored row major; V^T fragments come from
+// ds_read_b64_tr_b16 (transpose-on-read), so nothing is transposed on the way in.
+//
+// LDS layout of a [64][128] bf16 tile: 256-byte rows of sixteen 16-byte chunks, chunk c of row r stored at
+// chunk c ^ swz(r & 15), swz = swap of the two 2-bit halves.  The DMA writes LDS linearly in lane order, so
+// the swizzle is applied on the GLOBAL side (lane L of a load fetches the chunk that belongs at position L).
+// Measured on gfx950: ds_read_b128 over 32 consecutive rows ~220 B/clk/CU and the transpose reads
+// ~150 B/clk/CU with this function (row & 15 alone gives 219 / 61).
+#include "attn_common.hpp"
+
+namespace {
+
+constexpr int D = 128;
+constexpr int BN = 64;
+constexpr int WAVES = 8;
+constexpr int THREADS = WAVES * 64;
+constexpr int BM = WAVES * 32;
+constexpr int KS = D / 16;
+constexpr int DB = D / 32;
+constexpr int TILE_BYTES = BN * D * 2;       // 16 KiB
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K then V
+constexpr int STAGES = 3;
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+constexpr int LOADS_PER_TILE = 2 * TILE_BYTES / (WAVES * 1024);  // DMA instructions per wavefront per stage (4)
+
+
+__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+#define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define MLTS_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int N>
+__device__ __forceinline__ void wait_vm_and_barrier() {
+  // raw barrier: __syncthreads() would also wait for the DMA loads of the NEXT tiles (vmcnt(0))
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// LDS reads are issued through inline assembly with explicitly counted waits.  Reads the compiler knows about are
+// made to wait for every outstanding LDS-DMA load (it cannot tell the ring stages apart), which would drain
+// the prefetch of the next tiles in the middle of each tile.  The rule that keeps the counted waits safe whatever
+// the compiler interleaves: wait_lgkm<N>(regs) is only used when N or more LGKM operations of this code
+// were issued AFTER the reads that fill `regs`; LDS operations return in order, so those reads are done.
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+
+template <int OFF>
+__device__ __forceinline__ v4i32 lds_read_b128(uint32_t addr) {
+  v4i32 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ v2i32 lds_read_tr16_b64(uint32_t addr) {
+  v2i32 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32& a, v4i32& b, v4i32& c, v4i32& d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v2i32 (&x)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+               : "n"(N));
+}
+__device__ __forceinline__ bf16x8 as_frag(v4i32 x) { return __builtin_bit_cast(bf16x8, x); }
+__device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+}
+
+template <int MODE>
+__global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams p) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
+
+  // Longest (last) q-tiles first across the whole grid: with causal masks the work per q-tile varies 16:1 and
+  // this order keeps the tail short.  (Grouping a head's q-tiles on one XCD for L2 locality was measured: no gain
+  // without a mask, 14% slower with the causal mask because of the longer tail.)
+  const int nbh = p.B * p.Hq;
+  const int bid = blockIdx.x;
+  const int qt = p.nqt - 1 - bid / nbh;
+  const int bh = bid % nbh;
+  const int b = bh / p.Hq, hq = bh % p.Hq;
+  const int hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = qt * BM;
+  const int wq0 = q0 + wave * 32;
+  const int qrow = wq0 + l32;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
+  bf16_t* O = static_cast<bf16_t*>(p.o) + b * p.os[0] + hq * p.os[1];
+
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (qrow < p.Sq) {
+      qf[ks] = *reinterpret_cast<const bf16x8*>(Q + static_cast<int64_t>(qrow) * p.qs[2] + ks * 16 + hh * 8);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[ks][i] = static_cast<bf16_t>(0.f);
+    }
+  }
+  int qpos = 0, qseq = -1;
+  int4 wq_stats = make_int4(0, -1, 0, -1);
+  int4 bq_stats[BM / 64];
+  if (MODE == MLTS_MASK_DOC) {
+    if (qrow < p.Sq) {
+      qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qrow];
+      qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qrow];
+    }
+#pragma unroll
+    for (int w = 0; w < BM / 64; ++w) {
+      const int t = (q0 >> 6) + w;
+      bq_stats[w] = t < p.nq_stats ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
+    }
+    const int t = wq0 >> 6;
+    if (t < p.nq_stats) wq_stats = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t];
+  }
+
+  const int nkt = (p.Sk + BN - 1) / BN;
+  int j_end = nkt;
+  if (MODE == MLTS_MASK_CAUSAL) {
+    const int lim = min(q0 + BM, p.Sq) - 1 + p.causal_off;
+    j_end = lim < 0 ? 0 : min(nkt, lim / BN + 1);
+  }
+  const int wave_last_q = min(wq0 + 31, p.Sq - 1);
+  auto block_needs = [&](int j) -> bool {
+    if (MODE != MLTS_MASK_DOC) return true;
+    const int4 ks4 = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
+    bool need = false;
+#pragma unroll
+    for (int w = 0; w < BM / 64; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
+    return need;
+  };
+  auto next_tile = [&](int j) -> int {
+    while (j < j_end && !block_needs(j)) ++j;
+    return j;
+  };
+
+  // ---- DMA loader: this wavefront moves 1 KiB pieces 2w, 2w+1 of the K tile and of the V tile ----
+  // piece n holds rows 4n .. 4n+3; lane L -> row 4n + L/16, stored chunk L%16, source chunk (L%16) ^ swz(row)
+  int ld_row[2], ld_col[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int row = (wave * 2 + n) * 4 + (lane >> 4);
+    ld_row[n] = row;
+    ld_col[n] = ((lane & 15) ^ swz4(row & 15)) * 8;
+  }
+  auto issue_tile = [&](int j, int stage) {
+    const int kv0 = j * BN;
+    unsigned char* sbase = smem + stage * STAGE_BYTES;
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
+      const bf16_t* ksrc = K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n];
+      const bf16_t* vsrc = V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n];
+      __builtin_amdgcn_global_load_lds(MLTS_GLB(ksrc), MLTS_LDS(sbase + (wave * 2 + n) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(MLTS_GLB(vsrc), MLTS_LDS(sbase + TILE_BYTES + (wave * 2 + n) * 1024), 16, 0, 0);
+    }
+  };
+
+  // ---- per-lane LDS read offsets (tile invariant) ----
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
+  int koff[KS];   // K fragment (A operand of S^T): row l32 (+32 kb), chunk 2 ks + hh
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+  int voff[2][DB];  // V^T fragment halves: key row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4)
+#pragma unroll
+  for (int part = 0; part < 2; ++part) {
+    const int rlow = part * 8 + hh * 4 + (l16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
+      voff[part][db] = rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+    }
+  }
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // prologue: two tiles in flight
+  int j = next_tile(0);
+  int j1 = j < j_end ? next_tile(j + 1) : j_end;
+  if (j < j_end) issue_tile(j, 0);
+  if (j1 < j_end) issue_tile(j1, 1);
+  int stage = 0;
+  while (j < j_end) {
+    const int j2 = j1 < j_end ? next_tile(j1 + 1) : j_end;
+    if (j1 < j_end) wait_vm_and_barrier<LOADS_PER_TILE>();  // tile j has landed; tile j1 may still be in flight
+    else wait_vm_and_barrier<0>();
+    if (j2 < j_end) issue_tile(j2, stage >= 1 ? stage - 1 : 2);  // stage (s + 2) % 3: read last during the previous tile
+
+    const int kv0 = j * BN;
+    int cls = TILE_FULL;
+    if (MODE == MLTS_MASK_CAUSAL) {
+      if (kv0 > wave_last_q + p.causal_off) cls = TILE_SKIP;
+      else if (kv0 + BN - 1 > wq0 + p.causal_off) cls = TILE_MASKED;
+    } else if (MODE == MLTS_MASK_DOC) {
+      cls = classify_doc_tile(wq_stats, p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j]);
+    }
+    if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;
+    if (wq0 >= p.Sq) cls = TILE_SKIP;
+
+    if (cls != TILE_SKIP) {
+      const uint32_t sb = lds0 + stage * STAGE_BYTES;
+      uint32_t ka[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ka[ks] = sb + koff[ks];
+      f32x16 sacc[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
+      {
+        // sixteen K fragments in four groups of four, two groups in flight
+        v4i32 g0[4], g1[4];
+#define MLTS_KREAD4(dst, KB, KS0)                                   \
+  dst[0] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 0]);               \
+  dst[1] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 1]);               \
+  dst[2] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 2]);               \
+  dst[3] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 3]);
+#define MLTS_KMFMA4(src, KB, KS0)                                                                              \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) sacc[KB] =                                                     \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[i]), qf[(KS0) + i], sacc[KB], 0, 0, 0);
+        MLTS_KREAD4(g0, 0, 0)
+        MLTS_KREAD4(g1, 0, 4)
+        wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
+        MLTS_KMFMA4(g0, 0, 0)
+        MLTS_KREAD4(g0, 1, 0)
+        wait_lgkm<4>(g1[0], g1[1], g1[2], g1[3]);
+        MLTS_KMFMA4(g1, 0, 4)
+        MLTS_KREAD4(g1, 1, 4)
+        wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
+        MLTS_KMFMA4(g0, 1, 0)
+        wait_lgkm<0>(g1[0], g1[1], g1[2], g1[3]);
+        MLTS_KMFMA4(g1, 1, 4)
+#undef MLTS_KREAD4
+#undef MLTS_KMFMA4
+      }
+
+      if (cls == TILE_MASKED) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+            int kp[4], ksq[4];
+            if (MODE == MLTS_MASK_DOC) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int kj = kbase + r;
+                const bool ok = kj < p.Sk;
+                kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
+                ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
+              }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int kj = kbase + r;
+              bool vis = kj < p.Sk;
+              if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
+              if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+              if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
+            }
+          }
+        }
+      }
+
+      // online softmax; the running maximum is only raised when it grows by more than 2^8 (the result is
+      // exact either way: l and O carry the same stale scale), so the O rescale is rare after the first tiles
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+      const bool raise = mx > m_run + 8.0f;  // also true for the first visible tile (m_run = -inf)
+      if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+        const float m_new = raise ? mx : m_run;
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);  // 1 for lanes that do not raise; 0 from -inf
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
+      }
+      const float m_use = m_run == -INFINITY ? 0.f : m_run;
+      bf16x8 pf[4];
+      float ls = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float pv = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + i] * p.scale_log2 - m_use);
+            ls += pv;
+            pf[kb * 2 + t][i] = static_cast<bf16_t>(pv);
+          }
+      l_run += ls;
+
+      {
+        // V^T fragments of one 16-key step: eight transpose reads (4 head-dim blocks x 2 halves); two steps in flight
+        uint32_t va[2][DB];
+#pragma unroll
+        for (int part = 0; part < 2; ++part)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) va[part][db] = sb + voff[part][db];
+        v2i32 h0[8], h1[8];
+#define MLTS_VREAD8(dst, C)                                                                 \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                                       \
+    dst[2 * db] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[0][db]);                    \
+    dst[2 * db + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[1][db]);                \
+  }
+#define MLTS_VMFMA4(src, C)                                                                                     \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) oacc[db] =                                                  \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2 * db], src[2 * db + 1]), pf[C], oacc[db], 0, 0, 0);
+        MLTS_VREAD8(h0, 0)
+        MLTS_VREAD8(h1, 1)
+        wait_lgkm<8>(h0);
+        MLTS_VMFMA4(h0, 0)
+        MLTS_VREAD8(h0, 2)
+        wait_lgkm<8>(h1);
+        MLTS_VMFMA4(h1, 1)
+        MLTS_VREAD8(h1, 3)
+        wait_lgkm<8>(h0);
+        MLTS_VMFMA4(h0, 2)
+        wait_lgkm<0>(h1);
+        MLTS_VMFMA4(h1, 3)
+#undef MLTS_VREAD8
+#undef MLTS_VMFMA4
+      }
+    }
+    j = j1;
+    j1 = j2;
+    stage = stage == 2 ? 0 : stage + 1;
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+  if (qrow < p.Sq) {
+    if (hh == 0) {
+      p.lse[(static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow] =
+          l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+    }
+    bf16_t* orow = O + static_cast<int64_t>(qrow) * p.os[2];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(oacc[db][g * 4 + r] * inv);
+        *reinterpret_cast<bf16x4*>(orow + db * 32 + g * 8 + hh * 4) = w;
+      }
+    }
+  }
+}
+
+template <int MODE>
+int launch(AttnParams p, hipStream_t st) {
+  auto kern = attn_fwd_dma_kernel<MODE>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) {
+      mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      return MLTS_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  p.nqt = (p.Sq + BM - 1) / BM;
+  const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * p.Hq;
+  {
+    MltsKernelTimer timer("attn_fwd", st);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, p);
+  }
+  return mlts_check_launch("mlts_attn_fwd");
+}
+
+}  // namespace
+
+// Requires head_dim 128, Sk >= 1 and 16-byte aligned rows (checked by the caller).
+int mlts_attn_fwd_bf16_dma(const AttnParams& p, int mode, hipStream_t st) {
+  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(p, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(p, st);
+  return launch<MLTS_MASK_DOC>(p, st);
+}
