@@ -2,7 +2,7 @@
 //
 // Same math and register layouts as attn_fwd.hip (S^T = K Q^T, P in registers, O^T = V^T P^T, eight
 // wavefronts x 32 query rows), but K and V tiles travel global -> LDS with the 16-byte LDS-DMA loads
-// (global_load_lds_dwordx4: no staging registers, no ds_write, no VALU work) into a three-stage ring, so a
+// (global_load_lds_dwordx4: no staging registers, no ds_write, no VALU work) into a four-stage ring, so a
 // tile's loads are issued two tiles ahead of its use.  Tiles are stored row major; V^T fragments come from
 // ds_read_b64_tr_b16 (transpose-on-read), so nothing is transposed on the way in.
 //
@@ -24,7 +24,7 @@ constexpr int KS = D / 16;
 constexpr int DB = D / 32;
 constexpr int TILE_BYTES = BN * D * 2;       // 16 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K then V
-constexpr int STAGES = 3;
+constexpr int STAGES = 4;
 constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
 constexpr int LOADS_PER_TILE = 2 * TILE_BYTES / (WAVES * 1024);  // DMA instructions per wavefront per stage (4)
 
@@ -191,17 +191,81 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  // prologue: two tiles in flight
-  int j = next_tile(0);
-  int j1 = j < j_end ? next_tile(j + 1) : j_end;
-  if (j < j_end) issue_tile(j, 0);
-  if (j1 < j_end) issue_tile(j1, 1);
-  int stage = 0;
-  while (j < j_end) {
-    const int j2 = j1 < j_end ? next_tile(j1 + 1) : j_end;
-    if (j1 < j_end) wait_vm_and_barrier<LOADS_PER_TILE>();  // tile j has landed; tile j1 may still be in flight
+  // ---- tile pipeline ----
+  // Per wavefront the phases of the tile stream are ... PV(t-1) QK(t) | SM(t) PV(t) QK(t+1) | SM(t+1) ...: one block
+  // of MFMA work (PV of the previous tile, then QK of this one) and one block of VALU work (softmax).  A SIMD hosts
+  // two wavefronts of the workgroup, w and w + 4; the workgroup barrier sits before the MFMA block in w < 4 and
+  // before the VALU block in w >= 4, so that the two run half a tile apart and one does softmax while the other
+  // keeps the matrix cores busy.  sync() number k (k = 0, 1, ...) means "the k-th needed tile has landed everywhere";
+  // the load of tile k + 2 is issued right behind it into ring stage (k + 2) % 4, which held tile k - 2: the early
+  // wavefronts finished it two syncs ago, the late ones read its V before their QK(k - 1), i.e. before this sync.
+  const bool late = wave >= WAVES / 2;
+  int inflight = 0, istage = 0;
+  int ji = next_tile(0);
+  auto issue_next = [&]() {
+    if (ji < j_end) {
+      issue_tile(ji, istage);
+      istage = (istage + 1) & (STAGES - 1);
+      ji = next_tile(ji + 1);
+      ++inflight;
+    }
+  };
+  auto sync = [&]() {
+    if (inflight >= 2) wait_vm_and_barrier<LOADS_PER_TILE>();  // oldest tile landed; the next may still be in flight
     else wait_vm_and_barrier<0>();
-    if (j2 < j_end) issue_tile(j2, stage >= 1 ? stage - 1 : 2);  // stage (s + 2) % 3: read last during the previous tile
+    --inflight;
+    issue_next();
+  };
+  issue_next();
+  issue_next();
+
+  f32x16 sacc[2];
+  bf16x8 pf[4];
+  bool pv_pending = false;
+  int pv_stage = 0;
+
+  auto pv_phase = [&]() {
+      {
+        // V^T fragments of one 16-key step: eight transpose reads (4 head-dim blocks x 2 halves); two steps in flight
+        const uint32_t sb = lds0 + pv_stage * STAGE_BYTES;
+        uint32_t va[2][DB];
+#pragma unroll
+        for (int part = 0; part < 2; ++part)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) va[part][db] = sb + voff[part][db];
+        v2i32 h0[8], h1[8];
+#define MLTS_VREAD8(dst, C)                                                                 \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                                       \
+    dst[2 * db] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[0][db]);                    \
+    dst[2 * db + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[1][db]);                \
+  }
+#define MLTS_VMFMA4(src, C)                                                                                     \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) oacc[db] =                                                  \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2 * db], src[2 * db + 1]), pf[C], oacc[db], 0, 0, 0);
+        MLTS_VREAD8(h0, 0)
+        MLTS_VREAD8(h1, 1)
+        wait_lgkm<8>(h0);
+        MLTS_VMFMA4(h0, 0)
+        MLTS_VREAD8(h0, 2)
+        wait_lgkm<8>(h1);
+        MLTS_VMFMA4(h1, 1)
+        MLTS_VREAD8(h1, 3)
+        wait_lgkm<8>(h0);
+        MLTS_VMFMA4(h0, 2)
+        wait_lgkm<0>(h1);
+        MLTS_VMFMA4(h1, 3)
+#undef MLTS_VREAD8
+#undef MLTS_VMFMA4
+      }
+  };
+
+  int j = next_tile(0);
+  int stage = 0;
+  if (late && j < j_end) sync();
+  while (j < j_end) {
+    const int jn = next_tile(j + 1);
+    if (!late) sync();
+    if (pv_pending) pv_phase();
 
     const int kv0 = j * BN;
     int cls = TILE_FULL;
@@ -219,7 +283,6 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       uint32_t ka[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) ka[ks] = sb + koff[ks];
-      f32x16 sacc[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -251,6 +314,9 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 #undef MLTS_KMFMA4
       }
 
+    }
+    if (late && jn < j_end) sync();
+    if (cls != TILE_SKIP) {
       if (cls == TILE_MASKED) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -300,7 +366,6 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
           for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
       }
       const float m_use = m_run == -INFINITY ? 0.f : m_run;
-      bf16x8 pf[4];
       float ls = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
@@ -314,42 +379,13 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
           }
       l_run += ls;
 
-      {
-        // V^T fragments of one 16-key step: eight transpose reads (4 head-dim blocks x 2 halves); two steps in flight
-        uint32_t va[2][DB];
-#pragma unroll
-        for (int part = 0; part < 2; ++part)
-#pragma unroll
-          for (int db = 0; db < DB; ++db) va[part][db] = sb + voff[part][db];
-        v2i32 h0[8], h1[8];
-#define MLTS_VREAD8(dst, C)                                                                 \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                                       \
-    dst[2 * db] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[0][db]);                    \
-    dst[2 * db + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[1][db]);                \
-  }
-#define MLTS_VMFMA4(src, C)                                                                                     \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) oacc[db] =                                                  \
-      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2 * db], src[2 * db + 1]), pf[C], oacc[db], 0, 0, 0);
-        MLTS_VREAD8(h0, 0)
-        MLTS_VREAD8(h1, 1)
-        wait_lgkm<8>(h0);
-        MLTS_VMFMA4(h0, 0)
-        MLTS_VREAD8(h0, 2)
-        wait_lgkm<8>(h1);
-        MLTS_VMFMA4(h1, 1)
-        MLTS_VREAD8(h1, 3)
-        wait_lgkm<8>(h0);
-        MLTS_VMFMA4(h0, 2)
-        wait_lgkm<0>(h1);
-        MLTS_VMFMA4(h1, 3)
-#undef MLTS_VREAD8
-#undef MLTS_VMFMA4
-      }
     }
-    j = j1;
-    j1 = j2;
-    stage = stage == 2 ? 0 : stage + 1;
+    pv_pending = cls != TILE_SKIP;
+    pv_stage = stage;
+    j = jn;
+    stage = (stage + 1) & (STAGES - 1);
   }
+  if (pv_pending) pv_phase();
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
