@@ -23,6 +23,10 @@ import time
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
+# HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled
+# by the same counters over the --calibrate-traffic kernel (summary: profiles/attn_cfg2_hbm_traffic.md).  Counters
+# cannot be read from inside the timed run, so the figures are carried here and refreshed with the profile.
+MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 619.0e6, "attn_bwd_dkdv": 885.3e6, "attn_bwd_dq": 841.4e6}
 
 
 def parse_args():
@@ -32,6 +36,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-extra", action="store_true", help="only the headline attention workload")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--calibrate-traffic", action="store_true",
+                    help="only launch the streaming kernel of known size (mlts_scale over 1 GiB of fp32: 1 GiB read, "
+                         "1 GiB written per launch) that the FETCH_SIZE / WRITE_SIZE counters are scaled against")
     return ap.parse_args()
 
 
@@ -196,6 +203,14 @@ def main() -> int:
         print("bench.py needs a GPU: the HIP path has no CPU fallback.", file=sys.stderr)
         return 2
     dev = torch.device("cuda:0")
+    if args.calibrate_traffic:
+        x = torch.ones(1 << 28, device=dev)
+        for _ in range(3):
+            ops.scale_(x, 1.0001)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_kernel": "scale_kernel", "launches": 3, "read_bytes_per_launch": 1 << 30,
+                          "written_bytes_per_launch": 1 << 30}))
+        return 0
     sec, flops, kernels, kernel_flops = bench_attention(torch, ops, _lib, dev, args.steps, args.warmup)
     total_flops = flops["fwd"] + flops["bwd"]
     value = total_flops / sec / 1e12
@@ -217,7 +232,8 @@ def main() -> int:
         "config": {"workload": "causal self-attention fwd+bwd, B=4 H=16 S=4096 D=128, bf16 (configuration 2)",
                    "flops_per_step": total_flops, "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS},
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": dom["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": dom["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": dom["tflops"] / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(dominant),
                      "kernel_ms": dom["ms"], "algorithmic_flops_per_launch": kernel_flops[dominant]},
         "kernels": kernels,
     }
