@@ -393,18 +393,32 @@ int launch_bwd(const AttnBwdParams& bp, hipStream_t st) {
 
 int mlts_attn_bwd_dq_bf16(const AttnBwdParams& bp, int D, int mode, hipStream_t st);
 
+int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq);                          // attn_bwd_dma.hip
+int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);       // attn_bwd_dma.hip
+
+namespace {
+// tuning aid: MLTS_BWD_VARIANT=staged selects the register-staged dK/dV kernel for head_dim 128 as well
+bool use_dma_dkdv(int D) {
+  static const bool staged = [] {
+    const char* e = getenv("MLTS_BWD_VARIANT");
+    return e && e[0] == 's';
+  }();
+  return D == 128 && !staged;
+}
+}  // namespace
+
 int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32) {
-  (void)s;
   (void)accumulate_f32;
-  return 0;
+  return s->D == 128 ? mlts_attn_bwd_dkdv_dma_workspace(s->B, s->Hq, s->Sq) : 0;
 }
 
 int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
-  (void)workspace;
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   int rc;
-  if (D == 128) {
+  if (use_dma_dkdv(D)) {
+    rc = mlts_attn_bwd_dkdv_bf16_dma(bp, mode, workspace, st);
+  } else if (D == 128) {
     if (mode == MLTS_MASK_NONE) rc = launch_bwd<128, MLTS_MASK_NONE>(bp, st);
     else if (mode == MLTS_MASK_CAUSAL) rc = launch_bwd<128, MLTS_MASK_CAUSAL>(bp, st);
     else rc = launch_bwd<128, MLTS_MASK_DOC>(bp, st);
