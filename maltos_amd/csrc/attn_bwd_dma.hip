@@ -76,11 +76,15 @@ __device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
   return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
 }
 
+// lse2[i] = lse[i] * log2(e), +inf where the row saw no key; lse2[n] = +inf is the entry that query rows beyond
+// the end of the sequence are pointed at, so that their probabilities come out as exp2(s - inf) = 0 without a mask
 __global__ __launch_bounds__(256) void lse2_kernel(const float* __restrict__ lse, float* __restrict__ lse2, int64_t n) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (i < n) {
     const float l = lse[i];
     lse2[i] = l == -INFINITY ? INFINITY : l * kLog2e;
+  } else if (i == n) {
+    lse2[i] = INFINITY;
   }
 }
 
@@ -168,6 +172,7 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_dkdv_dma_kernel(const Att
     ld_row[n] = row;
     ld_col[n] = ((lane & 15) ^ swz4(row & 15)) * 8;
   }
+  const int64_t lse2_inf = static_cast<int64_t>(p.B) * p.Hq * p.Sq;  // index of the +inf entry
   auto issue_tile = [&](int it, int stage) {
     const int hq = hkv * group + it / span;
     const int q0 = (qt_begin + it % span) * BQ;
@@ -182,8 +187,9 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_dkdv_dma_kernel(const Att
       __builtin_amdgcn_global_load_lds(MLTS_GLB(qsrc), MLTS_LDS(sbase + (wave * 4 + n) * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(MLTS_GLB(dsrc), MLTS_LDS(sbase + TILE_BYTES + (wave * 4 + n) * 1024), 16, 0, 0);
     }
-    const int64_t soff = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + min(q0 + lane, p.Sq - 1);
-    const float* ssrc = ((wave & 1) ? bp.delta : lse2) + soff;
+    const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
+    const float* ssrc = (wave & 1) ? bp.delta + srow + min(q0 + lane, p.Sq - 1)
+                                   : lse2 + (q0 + lane < p.Sq ? srow + q0 + lane : lse2_inf);
     __builtin_amdgcn_global_load_lds(MLTS_GLB(ssrc), MLTS_LDS(sbase + STAT_OFF + (wave & 1) * (BQ * 4)), 4, 0, 0);
   };
 
@@ -228,9 +234,200 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_dkdv_dma_kernel(const Att
   issue_next();
   issue_next();
 
+  const int kj = wkv0 + l32;
+
+  // One (128-key, 64-query) tile for this wavefront's 32 keys, straight-line code (the masked and the unmasked form
+  // are separate instances so that nothing branches inside).  The matrix work is cut into sixteen groups of four
+  // MFMAs; the softmax arithmetic of query block 0 is written between the S/dP groups of query block 1, and that of
+  // block 1 between the first dV/dK groups, so that the one wavefront per SIMD has VALU work to issue while the
+  // matrix pipe is busy.  P and -dS stay in registers: lane = key (wkv0 + l32), accumulator register e <-> query
+  // 32 qb + 8 (e/4) + 4 hh + e%4, which is the A-operand layout of the dV/dK products.
+  auto process_tile = [&](auto masked_tag, const int q0, const int stage) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const uint32_t sb = lds0 + stage * STAGE_BYTES;
+    uint32_t ra[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
+    const uint32_t sa = sb + soff_lane;
+    uint32_t ta[2][DB];
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+
+    bf16x8 pfr[2][2], dsfr[2][2];
+    f32x16 sacc[2], dpacc[2];  // matrix-pipe accumulators (AGPRs in this kernel)
+    f32x16 sv[2], dv_[2];      // their copies in VGPRs for the softmax arithmetic
+    f32x4 lse4[2][4];
+    const int causal_t = kj - p.causal_off - q0 - hh * 4;
+
+    auto softmax_chunk = [&](auto qb_tag, auto g_tag) {  // four queries: rows 32 qb + 8 g + 4 hh .. +3
+      constexpr int qb = decltype(qb_tag)::value;
+      constexpr int g = decltype(g_tag)::value;
+      const int qrow = qb * 32 + g * 8 + hh * 4;
+      int qp4[4], qs4[4];
+      if (MASKED && MODE == MLTS_MASK_DOC) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int qi = q0 + qrow + r;
+          const bool ok = qi < p.Sq;
+          qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
+          qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
+        }
+      }
+      float pv[4], nds[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int e = g * 4 + r;
+        pv[r] = __builtin_amdgcn_exp2f(sv[qb][e] * p.scale_log2 - lse4[qb][g][r]);
+        if (MASKED) {
+          bool vis;
+          if (MODE == MLTS_MASK_CAUSAL) {
+            vis = causal_t <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
+          } else {
+            const int qi = q0 + qrow + r;
+            vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
+          }
+          if (!vis) pv[r] = 0.f;
+        }
+        nds[r] = pv[r] * dv_[qb][e];  // -dS
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pfr[qb][g >> 1][(g & 1) * 4 + r] = static_cast<bf16_t>(pv[r]);
+        dsfr[qb][g >> 1][(g & 1) * 4 + r] = static_cast<bf16_t>(nds[r]);
+      }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+
+#define MLTS_RREAD4(dst, QB, KS0)                                                  \
+  dst[0] = lds_read_b128<(QB) * 8192>(ra[(KS0)]);                                  \
+  dst[1] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 1]);                              \
+  dst[2] = lds_read_b128<TILE_BYTES + (QB) * 8192>(ra[(KS0)]);                     \
+  dst[3] = lds_read_b128<TILE_BYTES + (QB) * 8192>(ra[(KS0) + 1]);
+#define MLTS_SMFMA4(src, QB, KS0)                                                                                  \
+  sacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), kf[(KS0)], sacc[QB], 0, 0, 0);                \
+  dpacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2]), nvf[(KS0)], dpacc[QB], 0, 0, 0);             \
+  sacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), kf[(KS0) + 1], sacc[QB], 0, 0, 0);            \
+  dpacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[3]), nvf[(KS0) + 1], dpacc[QB], 0, 0, 0);
+#define MLTS_STAT_READ(st, QB)                                                    \
+  _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                 \
+    st[g] = lds_read_b128<(QB) * 128>(sa + g * 32);                               \
+    st[4 + g] = lds_read_b128<BQ * 4 + (QB) * 128>(sa + g * 32);                  \
+  }
+    // whole-vector casts below: casting a single element of an asm result is miscompiled (element 0 is broadcast)
+#define MLTS_STAT_USE(st, QB)                                                     \
+  _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                 \
+    lse4[QB][g] = __builtin_bit_cast(f32x4, st[g]);                               \
+    const f32x4 dl = __builtin_bit_cast(f32x4, st[4 + g]);                        \
+    _Pragma("unroll") for (int r = 0; r < 4; ++r) {                               \
+      sacc[QB][g * 4 + r] = 0.f;                                                  \
+      dpacc[QB][g * 4 + r] = dl[r];                                               \
+    }                                                                             \
+  }
+#define MLTS_TREAD8(dst, C, H)                                                                   \
+  _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
+    dst[4 * u + 0] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(ta[0][2 * (H) + u]);             \
+    dst[4 * u + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(ta[1][2 * (H) + u]);             \
+    dst[4 * u + 2] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H) + u]);                          \
+    dst[4 * u + 3] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H) + u]);                          \
+  }
+#define MLTS_TMFMA4(src, C, H)                                                                                        \
+  _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                                     \
+    dvacc[2 * (H) + u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pfr[(C) >> 1][(C) & 1], as_frag(src[4 * u], src[4 * u + 1]), \
+                                                                 dvacc[2 * (H) + u], 0, 0, 0);                        \
+    dkacc[2 * (H) + u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsfr[(C) >> 1][(C) & 1], as_frag(src[4 * u + 2], src[4 * u + 3]), \
+                                                                 dkacc[2 * (H) + u], 0, 0, 0);                        \
+  }
+    // the accumulators of one query block are copied out in one go, which frees their AGPRs for the next block
+#define MLTS_TO_VGPR(QB)                                         \
+  sv[QB] = sacc[QB];                                             \
+  dv_[QB] = dpacc[QB];                                           \
+  asm volatile("" : "+v"(sv[QB]), "+v"(dv_[QB]));
+    v4i32 st[8], g0[4], g1[4];
+    v2i32 h0[8], h1[8];
+    // phase A: S and delta - dO V^T of query block 0
+    MLTS_STAT_READ(st, 0)
+    MLTS_RREAD4(g0, 0, 0)
+    MLTS_RREAD4(g1, 0, 2)
+    wait_lgkm<8>(st);
+    MLTS_STAT_USE(st, 0)
+    wait_lgkm<4>(g0);
+    MLTS_SMFMA4(g0, 0, 0)
+    MLTS_RREAD4(g0, 0, 4)
+    wait_lgkm<4>(g1);
+    MLTS_SMFMA4(g1, 0, 2)
+    MLTS_RREAD4(g1, 0, 6)
+    wait_lgkm<4>(g0);
+    MLTS_SMFMA4(g0, 0, 4)
+    MLTS_STAT_READ(st, 1)
+    MLTS_RREAD4(g0, 1, 0)
+    wait_lgkm<12>(g1);
+    MLTS_SMFMA4(g1, 0, 6)
+    MLTS_RREAD4(g1, 1, 2)
+    MLTS_TO_VGPR(0)
+    // phase B: the same for query block 1, with the softmax of block 0 in between
+    wait_lgkm<8>(st);
+    MLTS_STAT_USE(st, 1)
+    wait_lgkm<4>(g0);
+    MLTS_SMFMA4(g0, 1, 0)
+    MLTS_RREAD4(g0, 1, 4)
+    softmax_chunk(I0{}, I0{});
+    wait_lgkm<4>(g1);
+    MLTS_SMFMA4(g1, 1, 2)
+    MLTS_RREAD4(g1, 1, 6)
+    softmax_chunk(I0{}, I1{});
+    wait_lgkm<4>(g0);
+    MLTS_SMFMA4(g0, 1, 4)
+    MLTS_TREAD8(h0, 0, 0)
+    softmax_chunk(I0{}, I2{});
+    wait_lgkm<8>(g1);
+    MLTS_SMFMA4(g1, 1, 6)
+    MLTS_TREAD8(h1, 0, 1)
+    softmax_chunk(I0{}, I3{});
+    MLTS_TO_VGPR(1)
+    // phase C: dV += P^T dO, -dK += (-dS)^T Q for the queries of block 0, with the softmax of block 1 in between
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, 0, 0)
+    MLTS_TREAD8(h0, 1, 0)
+    softmax_chunk(I1{}, I0{});
+    wait_lgkm<8>(h1);
+    MLTS_TMFMA4(h1, 0, 1)
+    MLTS_TREAD8(h1, 1, 1)
+    softmax_chunk(I1{}, I1{});
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, 1, 0)
+    MLTS_TREAD8(h0, 2, 0)
+    softmax_chunk(I1{}, I2{});
+    wait_lgkm<8>(h1);
+    MLTS_TMFMA4(h1, 1, 1)
+    MLTS_TREAD8(h1, 2, 1)
+    softmax_chunk(I1{}, I3{});
+    // phase D: the queries of block 1
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, 2, 0)
+    MLTS_TREAD8(h0, 3, 0)
+    wait_lgkm<8>(h1);
+    MLTS_TMFMA4(h1, 2, 1)
+    MLTS_TREAD8(h1, 3, 1)
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, 3, 0)
+    wait_lgkm<0>(h1);
+    MLTS_TMFMA4(h1, 3, 1)
+#undef MLTS_RREAD4
+#undef MLTS_SMFMA4
+#undef MLTS_STAT_READ
+#undef MLTS_STAT_USE
+#undef MLTS_TREAD8
+#undef MLTS_TMFMA4
+#undef MLTS_TO_VGPR
+  };
+
   int it = next_it(0);
   int stage = 0;
-  const int kj = wkv0 + l32;
   while (it < total_it) {
     const int qt = qt_begin + it % span;
     const int q0 = qt * BQ;
@@ -250,152 +447,16 @@ __global__ __launch_bounds__(THREADS, 1) void attn_bwd_dkdv_dma_kernel(const Att
     if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || q0 + BQ > p.Sq)) cls = TILE_MASKED;
     if (wkv0 >= p.Sk) cls = TILE_SKIP;
 
-    if (cls != TILE_SKIP) {
-      const uint32_t sb = lds0 + stage * STAGE_BYTES;
-      uint32_t ra[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
-      const uint32_t sa = sb + soff_lane;
-
-      // P and -dS in registers; lane = key (wkv0 + l32), register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4
-      bf16x8 pfr[2][2], dsfr[2][2];
-      f32x16 sacc[2], dpacc[2];
-      f32x4 lse4[2][4];
-
-      // ---- S = Q K^T and delta - dO V^T for both 32-query blocks ----
-#define MLTS_RREAD4(dst, QB, KS0)                                                  \
-  dst[0] = lds_read_b128<(QB) * 8192>(ra[(KS0)]);                                  \
-  dst[1] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 1]);                              \
-  dst[2] = lds_read_b128<TILE_BYTES + (QB) * 8192>(ra[(KS0)]);                     \
-  dst[3] = lds_read_b128<TILE_BYTES + (QB) * 8192>(ra[(KS0) + 1]);
-#define MLTS_SMFMA4(src, QB, KS0)                                                                                  \
-  sacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), kf[(KS0)], sacc[QB], 0, 0, 0);                \
-  dpacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2]), nvf[(KS0)], dpacc[QB], 0, 0, 0);             \
-  sacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), kf[(KS0) + 1], sacc[QB], 0, 0, 0);            \
-  dpacc[QB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[3]), nvf[(KS0) + 1], dpacc[QB], 0, 0, 0);
-#define MLTS_SDP_BLOCK(QB)                                                                        \
-  {                                                                                               \
-    v4i32 st[8];                                                                                  \
-    _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                               \
-      st[g] = lds_read_b128<(QB) * 128>(sa + g * 32);                                             \
-      st[4 + g] = lds_read_b128<BQ * 4 + (QB) * 128>(sa + g * 32);                                \
-    }                                                                                             \
-    v4i32 g0[4], g1[4];                                                                           \
-    MLTS_RREAD4(g0, QB, 0)                                                                        \
-    MLTS_RREAD4(g1, QB, 2)                                                                        \
-    wait_lgkm<8>(st);                                                                             \
-    _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                               \
-      lse4[QB][g] = __builtin_bit_cast(f32x4, st[g]);   /* whole-vector casts: casting one element */ \
-      const f32x4 dl = __builtin_bit_cast(f32x4, st[4 + g]);  /* of an asm result is miscompiled */  \
-      _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                             \
-        sacc[QB][g * 4 + r] = 0.f;                                                                \
-        dpacc[QB][g * 4 + r] = dl[r];                                                             \
-      }                                                                                           \
-    }                                                                                             \
-    wait_lgkm<4>(g0);                                                                             \
-    MLTS_SMFMA4(g0, QB, 0)                                                                        \
-    MLTS_RREAD4(g0, QB, 4)                                                                        \
-    wait_lgkm<4>(g1);                                                                             \
-    MLTS_SMFMA4(g1, QB, 2)                                                                        \
-    MLTS_RREAD4(g1, QB, 6)                                                                        \
-    wait_lgkm<4>(g0);                                                                             \
-    MLTS_SMFMA4(g0, QB, 4)                                                                        \
-    wait_lgkm<0>(g1);                                                                             \
-    MLTS_SMFMA4(g1, QB, 6)                                                                        \
-  }
-      MLTS_SDP_BLOCK(0)
-      MLTS_SDP_BLOCK(1)
-#undef MLTS_SDP_BLOCK
-#undef MLTS_SMFMA4
-#undef MLTS_RREAD4
-
-      auto softmax_bwd = [&](auto masked_tag, auto qb_tag) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        constexpr int qb = decltype(qb_tag)::value;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int qrow = qb * 32 + g * 8 + hh * 4;
-          int qp4[4], qs4[4];
-          if (MASKED && MODE == MLTS_MASK_DOC) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int qi = q0 + qrow + r;
-              const bool ok = qi < p.Sq;
-              qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
-              qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
-            }
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int e = g * 4 + r;
-            float pv = __builtin_amdgcn_exp2f(sacc[qb][e] * p.scale_log2 - lse4[qb][g][r]);
-            if (MASKED) {
-              const int qi = q0 + qrow + r;
-              bool vis = kj < p.Sk && qi < p.Sq;
-              if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qi + p.causal_off);
-              if (MODE == MLTS_MASK_DOC) vis = vis && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
-              if (!vis) pv = 0.f;
-            }
-            const float ndsv = pv * dpacc[qb][e];  // -dS
-            pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
-            dsfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(ndsv);
-          }
-        }
-      };
-
-      // ---- dV += P^T dO, -dK += (-dS)^T Q: per 16-query step c and pair of head-dim blocks, eight transpose reads ----
-      uint32_t ta[2][DB];
-#pragma unroll
-      for (int part = 0; part < 2; ++part)
-#pragma unroll
-        for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
-#define MLTS_TREAD8(dst, C, H)                                                                   \
-  _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                \
-    dst[4 * u + 0] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(ta[0][2 * (H) + u]);             \
-    dst[4 * u + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(ta[1][2 * (H) + u]);             \
-    dst[4 * u + 2] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H) + u]);                          \
-    dst[4 * u + 3] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H) + u]);                          \
-  }
-#define MLTS_TMFMA4(src, C, H)                                                                                        \
-  _Pragma("unroll") for (int u = 0; u < 2; ++u) {                                                                     \
-    dvacc[2 * (H) + u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pfr[(C) >> 1][(C) & 1], as_frag(src[4 * u], src[4 * u + 1]), \
-                                                                 dvacc[2 * (H) + u], 0, 0, 0);                        \
-    dkacc[2 * (H) + u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsfr[(C) >> 1][(C) & 1], as_frag(src[4 * u + 2], src[4 * u + 3]), \
-                                                                 dkacc[2 * (H) + u], 0, 0, 0);                        \
-  }
-      {
-        v2i32 h0[8], h1[8];
-        MLTS_TREAD8(h0, 0, 0)
-        MLTS_TREAD8(h1, 0, 1)
-        if (cls == TILE_MASKED) softmax_bwd(std::true_type{}, std::integral_constant<int, 0>{});
-        else softmax_bwd(std::false_type{}, std::integral_constant<int, 0>{});
-        wait_lgkm<8>(h0);
-        MLTS_TMFMA4(h0, 0, 0)
-        MLTS_TREAD8(h0, 1, 0)
-        wait_lgkm<8>(h1);
-        MLTS_TMFMA4(h1, 0, 1)
-        MLTS_TREAD8(h1, 1, 1)
-        wait_lgkm<8>(h0);
-        MLTS_TMFMA4(h0, 1, 0)
-        MLTS_TREAD8(h0, 2, 0)
-        wait_lgkm<8>(h1);
-        MLTS_TMFMA4(h1, 1, 1)
-        MLTS_TREAD8(h1, 2, 1)
-        if (cls == TILE_MASKED) softmax_bwd(std::true_type{}, std::integral_constant<int, 1>{});
-        else softmax_bwd(std::false_type{}, std::integral_constant<int, 1>{});
-        wait_lgkm<8>(h0);
-        MLTS_TMFMA4(h0, 2, 0)
-        MLTS_TREAD8(h0, 3, 0)
-        wait_lgkm<8>(h1);
-        MLTS_TMFMA4(h1, 2, 1)
-        MLTS_TREAD8(h1, 3, 1)
-        wait_lgkm<8>(h0);
-        MLTS_TMFMA4(h0, 3, 0)
-        wait_lgkm<0>(h1);
-        MLTS_TMFMA4(h1, 3, 1)
-      }
-#undef MLTS_TREAD8
-#undef MLTS_TMFMA4
+    // one instance of the tile body per mask mode where possible (two instances in one loop make the register
+    // allocator move the accumulators at every block boundary): without a mask nothing needs masking (keys past Sk
+    // are never stored, queries past Sq have lse2 = +inf), the causal comparison is cheap enough to be always on
+    if (MODE == MLTS_MASK_NONE) {
+      if (cls != TILE_SKIP) process_tile(std::false_type{}, q0, stage);
+    } else if (MODE == MLTS_MASK_CAUSAL) {
+      if (cls != TILE_SKIP) process_tile(std::true_type{}, q0, stage);
+    } else {
+      if (cls == TILE_FULL) process_tile(std::false_type{}, q0, stage);
+      else if (cls == TILE_MASKED) process_tile(std::true_type{}, q0, stage);
     }
     it = next_it(it + 1);
     stage = stage == STAGES - 1 ? 0 : stage + 1;
@@ -446,15 +507,15 @@ int launch(const AttnBwdParams& bp, const float* lse2, hipStream_t st) {
 
 }  // namespace
 
-int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq) { return ((B * Hq * Sq * 4 + 255) / 256) * 256; }
+int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq) { return (((B * Hq * Sq + 1) * 4 + 255) / 256) * 256; }
 
-// head_dim 128, Sq >= 1, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq floats.
+// head_dim 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
 int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   float* lse2 = static_cast<float*>(workspace);
   const int64_t n = static_cast<int64_t>(p.B) * p.Hq * p.Sq;
-  if (n > 0) hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, p.lse, lse2, n);
+  hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 256) / 256)), dim3(256), 0, st, p.lse, lse2, n);
   if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(bp, lse2, st);
   if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(bp, lse2, st);
   return launch<MLTS_MASK_DOC>(bp, lse2, st);
