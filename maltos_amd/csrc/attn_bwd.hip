@@ -396,14 +396,19 @@ int mlts_attn_bwd_dq_bf16(const AttnBwdParams& bp, int D, int mode, hipStream_t 
 int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq);                          // attn_bwd_dma.hip
 int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);       // attn_bwd_dma.hip
 
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);     // attn_bwd_split.hip
+
 namespace {
-// tuning aid: MLTS_BWD_VARIANT=staged selects the register-staged dK/dV kernel for head_dim 128 as well
-bool use_dma_dkdv(int D) {
-  static const bool staged = [] {
+// dK/dV kernel for head_dim 128: the two-role kernel by default; tuning aid MLTS_BWD_VARIANT = "staged" (register
+// staged tiles, the head_dim 64 kernel) or "dma" (one role, one wavefront per SIMD) selects the earlier forms
+int dkdv_variant(int D) {
+  static const int v = [] {
     const char* e = getenv("MLTS_BWD_VARIANT");
-    return e && e[0] == 's';
+    if (e && e[0] == 's') return 0;
+    if (e && e[0] == 'd') return 1;
+    return 2;
   }();
-  return D == 128 && !staged;
+  return D == 128 ? v : 0;
 }
 }  // namespace
 
@@ -416,7 +421,9 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   int rc;
-  if (use_dma_dkdv(D)) {
+  if (dkdv_variant(D) == 2) {
+    rc = mlts_attn_bwd_dkdv_bf16_split(bp, mode, workspace, st);
+  } else if (dkdv_variant(D) == 1) {
     rc = mlts_attn_bwd_dkdv_bf16_dma(bp, mode, workspace, st);
   } else if (D == 128) {
     if (mode == MLTS_MASK_NONE) rc = launch_bwd<128, MLTS_MASK_NONE>(bp, st);

@@ -1,0 +1,565 @@
+// Attention backward, dK and dV, head_dim 128, bf16: two-role workgroup.
+//
+// A workgroup owns 128 keys of one (batch, kv head) and walks the 64-row query tiles that can see them (all
+// query heads of the GQA group), as attn_bwd.hip does, but its EIGHT wavefronts come in two roles per 32-key
+// block kb = wave % 4:
+//     role 0 (wave < 4):   S = Q K^T,  P = exp2(S c - lse2)  ->  dV += P^T dO      and hands P (bf16) over in LDS
+//     role 1 (wave >= 4):  delta - dO V^T,  -dS = P (delta - dO V^T)  ->  -dK += (-dS)^T Q     one tile behind
+// Each role keeps one operand (K or -V) and one accumulator (dV or dK) in registers, so a wavefront fits in
+// 256 registers, two wavefronts share a SIMD, the matrix instructions take plain VGPR accumulators (no AGPR
+// copies around the softmax arithmetic) and the hardware overlaps one wavefront's VALU work with the other's
+// matrix work.  The two GEMMs of a role read different LDS operands, so the split costs no extra LDS traffic
+// beyond the 4 KiB of P per tile and key block.
+//
+// Memory pipeline: Q/dO tiles and the per-row statistics (lse2 = lse log2 e, delta) are fetched into registers right
+// behind the barrier of tile k and written to a three-stage LDS ring after the work on tile k (role 1 still reads
+// tile k - 1), row major with the chunk swizzle of attn_fwd_dma.hip; transposed operands come from
+// ds_read_b64_tr_b16; LDS accesses are issued through inline assembly with counted waits; delta is folded into
+// the dP accumulator and V is negated.
+#include "attn_common.hpp"
+#include <type_traits>
+
+namespace {
+
+constexpr int D = 128;
+constexpr int BKV = 128;
+constexpr int BQ = 64;
+constexpr int WAVES = 8;
+constexpr int THREADS = WAVES * 64;
+constexpr int KS = D / 16;
+constexpr int DB = D / 32;
+constexpr int TILE_BYTES = BQ * D * 2;          // 16 KiB
+constexpr int STAT_OFF = 2 * TILE_BYTES;        // lse2[64] then delta[64], fp32
+constexpr int STAGE_BYTES = STAT_OFF + 2 * BQ * 4;
+constexpr int STAGES = 3;
+constexpr int PBUF_OFF = STAGES * STAGE_BYTES;  // P hand-over: [2 buffers][4 key blocks][4 fragments][64 lanes] x 16 B
+constexpr int PBUF_BYTES = 4 * 64 * 16;
+constexpr int LDS_BYTES = PBUF_OFF + 2 * 4 * PBUF_BYTES;
+
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+#define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define MLTS_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// every LDS access of this wavefront has completed, then the workgroup barrier
+__device__ __forceinline__ void drain_and_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int OFF>
+__device__ __forceinline__ v4i32 lds_read_b128(uint32_t addr) {
+  v4i32 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ v2i32 lds_read_tr16_b64(uint32_t addr) {
+  v2i32 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write_b128(uint32_t addr, v4i32 x) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(x), "n"(OFF));
+}
+// wait_lgkm<N>(regs): only used when N or more LGKM operations of this code were issued after the reads into regs
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+               : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v2i32 (&x)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+               : "n"(N));
+}
+__device__ __forceinline__ bf16x8 as_frag(v4i32 x) { return __builtin_bit_cast(bf16x8, x); }
+__device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+}
+
+// lse2[i] = lse[i] * log2(e), +inf where the row saw no key; lse2[n] = +inf is the entry that query rows beyond
+// the end of the sequence are pointed at, so that their probabilities come out as exp2(s - inf) = 0 without a mask
+__global__ __launch_bounds__(256) void lse2_kernel(const float* __restrict__ lse, float* __restrict__ lse2, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n) {
+    const float l = lse[i];
+    lse2[i] = l == -INFINITY ? INFINITY : l * kLog2e;
+  } else if (i == n) {
+    lse2[i] = INFINITY;
+  }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const AttnBwdParams bp, const float* __restrict__ lse2) {
+  const AttnParams& p = bp.a;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
+  const int role = wave >> 2, kb = wave & 3;
+
+  const int nbh = p.B * p.Hkv;
+  const int bid = blockIdx.x;
+  const int kt = bid / nbh;  // key tile; low tiles see the most queries under a causal mask and go first
+  const int bh = bid % nbh;
+  const int b = bh / p.Hkv, hkv = bh % p.Hkv;
+  const int group = p.Hq / p.Hkv;
+  const int kv0 = kt * BKV;
+  const int wkv0 = kv0 + kb * 32;
+  const int kj = wkv0 + l32;
+
+  // ---- this wavefront's stationary operand (B operand of its first GEMM): K for role 0, -V for role 1 ----
+  bf16x8 kvf[KS];
+  {
+    const bf16_t* src = role == 0 ? static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1] + static_cast<int64_t>(kj) * p.ks[2]
+                                  : static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1] + static_cast<int64_t>(kj) * p.vs[2];
+    const int flip = role == 0 ? 0 : static_cast<int>(0x80008000u);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      v4i32 x = {0, 0, 0, 0};
+      if (kj < p.Sk) x = *reinterpret_cast<const v4i32*>(src + ks * 16 + hh * 8);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] ^= flip;
+      kvf[ks] = as_frag(x);
+    }
+  }
+
+  // ---- query-tile range ----
+  const int nqt = (p.Sq + BQ - 1) / BQ;
+  int qt_begin = 0;
+  if (MODE == MLTS_MASK_CAUSAL) {
+    const int first_q = kv0 - p.causal_off;  // first query that sees key kv0
+    qt_begin = first_q <= 0 ? 0 : first_q / BQ;
+  }
+  const int span = qt_begin < nqt ? nqt - qt_begin : 0;
+  const int total_it = span * group;
+
+  int4 kstats[2];
+  if (MODE == MLTS_MASK_DOC) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int t = (kv0 >> 6) + i;
+      kstats[i] = t < p.nk_stats ? p.k_stats[static_cast<int64_t>(b) * p.nk_stats + t] : make_int4(0x7fffffff, 0, 0, -2);
+    }
+  }
+  const int4 wk_stats = MODE == MLTS_MASK_DOC ? ((kb >> 1) ? kstats[1] : kstats[0]) : make_int4(0, 0, 0, 0);
+  int kpos = 0, kseq = -2;
+  if (MODE == MLTS_MASK_DOC && kj < p.Sk) {
+    kpos = p.k_pos[static_cast<int64_t>(b) * p.Sk + kj];
+    kseq = p.k_seq[static_cast<int64_t>(b) * p.Sk + kj];
+  }
+  auto block_needs = [&](int it) -> bool {
+    if (MODE != MLTS_MASK_DOC) return true;
+    const int qt = qt_begin + it % span;
+    const int4 qs4 = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt];
+    return classify_doc_tile(qs4, kstats[0]) != TILE_SKIP || classify_doc_tile(qs4, kstats[1]) != TILE_SKIP;
+  };
+  auto next_it = [&](int it) -> int {
+    while (it < total_it && !block_needs(it)) ++it;
+    return it;
+  };
+  auto classify = [&](int it) -> int {  // for this wavefront's 32 keys; identical in both roles of a key block
+    const int qt = qt_begin + it % span;
+    const int q0 = qt * BQ;
+    int cls = TILE_FULL;
+    if (MODE == MLTS_MASK_CAUSAL) {
+      const int last_q = min(q0 + BQ, p.Sq) - 1;
+      if (wkv0 > last_q + p.causal_off) cls = TILE_SKIP;
+      else if (wkv0 + 31 > q0 + p.causal_off) cls = TILE_MASKED;
+    } else if (MODE == MLTS_MASK_DOC) {
+      cls = classify_doc_tile(p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt], wk_stats);
+    }
+    if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || q0 + BQ > p.Sq)) cls = TILE_MASKED;
+    if (wkv0 >= p.Sk) cls = TILE_SKIP;
+    return cls;
+  };
+
+  // ---- tile loader.  Measured on gfx950: an LDS-DMA load keeps the LDS busy for about 27 cycles per KiB while its
+  // data arrives (3-4 times a ds_write_b128 of the same data) and ds_read streams of the whole CU stall meanwhile, and
+  // this kernel is bound by LDS time.  So the next tile is fetched into registers right behind the barrier (64 bytes
+  // per thread: chunks t and t + 512 of the Q tile and of the dO tile, chunk c = row c/16, stored 16-byte slot c%16,
+  // source slot (c%16) ^ swz(row)) and written to LDS with ds_write_b128 after this tile's work.  Threads 0..127 also
+  // carry the 64 + 64 row statistics (lse2, delta). ----
+  const int64_t lse2_inf = static_cast<int64_t>(p.B) * p.Hq * p.Sq;  // index of the +inf entry
+  int ld_row[2], ld_col[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int c = tid + n * THREADS;
+    ld_row[n] = c >> 4;
+    ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+  }
+  v4i32 stg_q[2], stg_d[2];
+  float stg_s = 0.f;
+  const uint32_t lds0_ = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
+  auto stage_load = [&](int it) {
+    const int hq = hkv * group + it / span;
+    const int q0 = (qt_begin + it % span) * BQ;
+    const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
+    const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1];
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int r = min(q0 + ld_row[n], p.Sq - 1);  // rows past the end repeat the last query; their lse2 is +inf
+      stg_q[n] = *reinterpret_cast<const v4i32*>(Q + static_cast<int64_t>(r) * p.qs[2] + ld_col[n]);
+      stg_d[n] = *reinterpret_cast<const v4i32*>(dO + static_cast<int64_t>(r) * bp.dos[2] + ld_col[n]);
+    }
+    if (tid < 2 * BQ) {
+      const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
+      const int r = q0 + (tid & (BQ - 1));
+      stg_s = tid < BQ ? lse2[r < p.Sq ? srow + r : lse2_inf] : bp.delta[srow + min(r, p.Sq - 1)];
+    }
+  };
+  const uint32_t stg_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem))) + tid * 16;
+  auto stage_store = [&](int stage) {
+    const uint32_t a = stg_lane + stage * STAGE_BYTES;
+    lds_write_b128<0>(a, stg_q[0]);
+    lds_write_b128<THREADS * 16>(a, stg_q[1]);
+    lds_write_b128<TILE_BYTES>(a, stg_d[0]);
+    lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_d[1]);
+    if (tid < 2 * BQ)
+      asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(lds0_ + stage * STAGE_BYTES + tid * 4), "v"(stg_s), "n"(STAT_OFF));
+  };
+
+  // ---- per-lane LDS offsets (tile invariant) ----
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
+  int roff[KS];  // row-major fragment (A operand): row l32 (+32 qb), chunk 2 ks + hh; role 0 reads Q, role 1 dO
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    roff[ks] = role * TILE_BYTES + l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+  int toff[2][DB];  // transposed fragment halves: query row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16)
+                    // + 4 (l16%4); role 0 reads dO^T, role 1 Q^T
+#pragma unroll
+  for (int part = 0; part < 2; ++part) {
+    const int rlow = part * 8 + hh * 4 + (l16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
+      toff[part][db] = (1 - role) * TILE_BYTES + rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+    }
+  }
+  // statistics of rows 32 qb + 8 g + 4 hh .. +3: role 0 reads lse2, role 1 delta
+  const int soff_lane = STAT_OFF + role * (BQ * 4) + hh * 16;
+  const uint32_t pbuf_lane = lds0 + PBUF_OFF + kb * PBUF_BYTES + lane * 16;
+
+  f32x16 acc[DB];  // dV (role 0) or -dK / scale (role 1): register e <-> key wkv0 + 8 (e/4) + 4 hh + e%4, lane -> column
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
+
+#define MLTS_RREAD4(dst, QB, KS0)                          \
+  dst[0] = lds_read_b128<(QB) * 8192>(ra[(KS0)]);          \
+  dst[1] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 1]);      \
+  dst[2] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 2]);      \
+  dst[3] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 3]);
+#define MLTS_RMFMA4(src, ACC, KS0)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) ACC =                                                 \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[i]), kvf[(KS0) + i], ACC, 0, 0, 0);
+#define MLTS_TREAD8(dst, C)                                                  \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                        \
+    dst[2 * db] = lds_read_tr16_b64<(C) * 4096>(ta[0][db]);                  \
+    dst[2 * db + 1] = lds_read_tr16_b64<(C) * 4096>(ta[1][db]);              \
+  }
+#define MLTS_TMFMA4(src, AFRAG)                                                                                  \
+  _Pragma("unroll") for (int db = 0; db < DB; ++db) acc[db] =                                                    \
+      __builtin_amdgcn_mfma_f32_32x32x16_bf16(AFRAG, as_frag(src[2 * db], src[2 * db + 1]), acc[db], 0, 0, 0);
+
+  // ---- role 0: one tile.  lane = key, accumulator register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4 ----
+  auto role0_tile = [&](auto masked_tag, const int q0, const int stage, const int pbuf) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const uint32_t sb = lds0 + stage * STAGE_BYTES;
+    uint32_t ra[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
+    const uint32_t sa = sb + soff_lane;
+    uint32_t ta[2][DB];
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+    const int causal_t = kj - p.causal_off - q0 - hh * 4;
+
+    bf16x8 pfr[2][2];
+    auto softmax = [&](auto qb_tag, const f32x16& s, const f32x4 (&lse4)[4]) {
+      constexpr int qb = decltype(qb_tag)::value;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int qrow = qb * 32 + g * 8 + hh * 4;
+        int qp4[4], qs4[4];
+        if (MASKED && MODE == MLTS_MASK_DOC) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int qi = q0 + qrow + r;
+            const bool ok = qi < p.Sq;
+            qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
+            qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int e = g * 4 + r;
+          float pv = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse4[g][r]);
+          if (MASKED) {
+            bool vis;
+            if (MODE == MLTS_MASK_CAUSAL) {
+              vis = causal_t <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
+            } else {
+              const int qi = q0 + qrow + r;
+              vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
+            }
+            if (!vis) pv = 0.f;
+          }
+          pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
+        }
+      }
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+
+    v4i32 st0[4], st1[4], g0[4], g1[4];
+    v2i32 h0[8], h1[8];
+    f32x16 s0, s1;
+    f32x4 lse4[4];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s0[e] = 0.f;
+      s1[e] = 0.f;
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) st0[g] = lds_read_b128<0>(sa + g * 32);
+    MLTS_RREAD4(g0, 0, 0)
+    MLTS_RREAD4(g1, 0, 4)
+    wait_lgkm<8>(st0);
+    wait_lgkm<4>(g0);
+    MLTS_RMFMA4(g0, s0, 0)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) st1[g] = lds_read_b128<128>(sa + g * 32);
+    MLTS_RREAD4(g0, 1, 0)
+    wait_lgkm<8>(g1);
+    MLTS_RMFMA4(g1, s0, 4)
+    MLTS_RREAD4(g1, 1, 4)
+    wait_lgkm<8>(st1);
+    wait_lgkm<4>(g0);
+    MLTS_RMFMA4(g0, s1, 0)
+    MLTS_TREAD8(h0, 0)
+    // whole-vector casts: casting a single element of an asm result is miscompiled (element 0 is broadcast)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
+    softmax(I0{}, s0, lse4);
+    wait_lgkm<8>(g1);
+    MLTS_RMFMA4(g1, s1, 4)
+    MLTS_TREAD8(h1, 1)
+    lds_write_b128<0>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][0]));
+    lds_write_b128<1024>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][1]));
+    wait_lgkm<10>(h0);
+    MLTS_TMFMA4(h0, pfr[0][0])
+    MLTS_TREAD8(h0, 2)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
+    softmax(I1{}, s1, lse4);
+    wait_lgkm<8>(h1);
+    MLTS_TMFMA4(h1, pfr[0][1])
+    MLTS_TREAD8(h1, 3)
+    lds_write_b128<2048>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][0]));
+    lds_write_b128<3072>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][1]));
+    wait_lgkm<10>(h0);
+    MLTS_TMFMA4(h0, pfr[1][0])
+    wait_lgkm<0>(h1);
+    MLTS_TMFMA4(h1, pfr[1][1])
+  };
+
+  // ---- role 1, first half of a tile: dp = delta - dO V^T (kept in registers until P arrives) ----
+  f32x16 dp0, dp1;
+  auto role1_dp = [&](const int stage) {
+    const uint32_t sb = lds0 + stage * STAGE_BYTES;
+    uint32_t ra[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
+    const uint32_t sa = sb + soff_lane;
+    v4i32 st[8], g0[4], g1[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      st[g] = lds_read_b128<0>(sa + g * 32);
+      st[4 + g] = lds_read_b128<128>(sa + g * 32);
+    }
+    MLTS_RREAD4(g0, 0, 0)
+    MLTS_RREAD4(g1, 0, 4)
+    wait_lgkm<8>(st);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 d0 = __builtin_bit_cast(f32x4, st[g]);
+      const f32x4 d1 = __builtin_bit_cast(f32x4, st[4 + g]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        dp0[g * 4 + r] = d0[r];
+        dp1[g * 4 + r] = d1[r];
+      }
+    }
+    wait_lgkm<4>(g0);
+    MLTS_RMFMA4(g0, dp0, 0)
+    MLTS_RREAD4(g0, 1, 0)
+    wait_lgkm<4>(g1);
+    MLTS_RMFMA4(g1, dp0, 4)
+    MLTS_RREAD4(g1, 1, 4)
+    wait_lgkm<4>(g0);
+    MLTS_RMFMA4(g0, dp1, 0)
+    wait_lgkm<0>(g1);
+    MLTS_RMFMA4(g1, dp1, 4)
+  };
+  // ---- role 1, second half (one barrier later): -dS = P dp, -dK += (-dS)^T Q ----
+  auto role1_dk = [&](const int stage, const int pbuf) {
+    const uint32_t sb = lds0 + stage * STAGE_BYTES;
+    uint32_t ta[2][DB];
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+    v4i32 pp[4];
+    v2i32 h0[8], h1[8];
+    pp[0] = lds_read_b128<0>(pbuf_lane + pbuf);
+    pp[1] = lds_read_b128<1024>(pbuf_lane + pbuf);
+    pp[2] = lds_read_b128<2048>(pbuf_lane + pbuf);
+    pp[3] = lds_read_b128<3072>(pbuf_lane + pbuf);
+    MLTS_TREAD8(h0, 0)
+    MLTS_TREAD8(h1, 1)
+    wait_lgkm<15>(pp);  // 16 reads follow; the counter field holds at most 15
+    bf16x8 dsfr[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int pw = pp[f][w];  // two bf16 probabilities
+        const float plo = __builtin_bit_cast(float, pw << 16);
+        const float phi = __builtin_bit_cast(float, pw & static_cast<int>(0xffff0000u));
+        const float dlo = (f >> 1) ? dp1[(f & 1) * 8 + 2 * w] : dp0[(f & 1) * 8 + 2 * w];
+        const float dhi = (f >> 1) ? dp1[(f & 1) * 8 + 2 * w + 1] : dp0[(f & 1) * 8 + 2 * w + 1];
+        dsfr[f][2 * w] = static_cast<bf16_t>(plo * dlo);
+        dsfr[f][2 * w + 1] = static_cast<bf16_t>(phi * dhi);
+      }
+    }
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, dsfr[0])
+    MLTS_TREAD8(h0, 2)
+    wait_lgkm<8>(h1);
+    MLTS_TMFMA4(h1, dsfr[1])
+    MLTS_TREAD8(h1, 3)
+    wait_lgkm<8>(h0);
+    MLTS_TMFMA4(h0, dsfr[2])
+    wait_lgkm<0>(h1);
+    MLTS_TMFMA4(h1, dsfr[3])
+  };
+#undef MLTS_RREAD4
+#undef MLTS_RMFMA4
+#undef MLTS_TREAD8
+#undef MLTS_TMFMA4
+
+  // ---- tile loop, one instance per role (so that the state of one role is not live in the other's code).
+  // Barrier k: tile k is in LDS and role 0 has handed over P of tile k - 1.  Tile k + 1 is fetched behind it and
+  // stored into stage (k + 1) % 3, which held tile k - 2 (role 1 finished it before this barrier). ----
+  auto tile_loop = [&](auto role_tag) {
+    constexpr int ROLE = decltype(role_tag)::value;
+    int it = next_it(0);
+    if (it < total_it) {
+      stage_load(it);
+      stage_store(0);
+    }
+    int stage = 0, k = 0;
+    bool prev_active = false;
+    int prev_stage = 0;
+    while (it < total_it) {
+      const int itn = next_it(it + 1);
+      drain_and_barrier();
+      if (itn < total_it) stage_load(itn);
+      const int q0 = (qt_begin + it % span) * BQ;
+      const int cls = classify(it);
+      const int pbuf = (k & 1) * (4 * PBUF_BYTES);
+      if (ROLE == 0) {
+        // one instance of the tile body per mask mode where possible: without a mask nothing needs masking (keys
+        // past Sk are never stored, queries past Sq have lse2 = +inf), the causal comparison is cheap enough to be
+        // always on
+        if (MODE == MLTS_MASK_NONE) {
+          if (cls != TILE_SKIP) role0_tile(std::false_type{}, q0, stage, pbuf);
+        } else if (MODE == MLTS_MASK_CAUSAL) {
+          if (cls != TILE_SKIP) role0_tile(std::true_type{}, q0, stage, pbuf);
+        } else {
+          if (cls == TILE_FULL) role0_tile(std::false_type{}, q0, stage, pbuf);
+          else if (cls == TILE_MASKED) role0_tile(std::true_type{}, q0, stage, pbuf);
+        }
+      } else {
+        if (prev_active) role1_dk(prev_stage, pbuf ^ (4 * PBUF_BYTES));
+        if (cls != TILE_SKIP) role1_dp(stage);
+      }
+      if (itn < total_it) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
+      prev_active = cls != TILE_SKIP;
+      prev_stage = stage;
+      it = itn;
+      stage = stage == STAGES - 1 ? 0 : stage + 1;
+      ++k;
+    }
+    drain_and_barrier();
+    if (ROLE == 1 && prev_active) role1_dk(prev_stage, ((k - 1) & 1) * (4 * PBUF_BYTES));
+  };
+  if (role == 0) tile_loop(std::integral_constant<int, 0>{});
+  else tile_loop(std::integral_constant<int, 1>{});
+
+  // ---- write dV (role 0) or dK (role 1) ----
+  {
+    const float oscale = role == 0 ? 1.0f : -p.scale;  // role 1 holds -dS^T Q
+    void* optr = role == 0 ? bp.dv : bp.dk;
+    const int64_t* os = role == 0 ? bp.dvs : bp.dks;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int d = db * 32 + l32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
+        if (row < p.Sk) {
+          const int64_t o = b * os[0] + hkv * os[1] + static_cast<int64_t>(row) * os[2] + d;
+          if (bp.accumulate_f32) static_cast<float*>(optr)[o] += acc[db][e] * oscale;
+          else static_cast<bf16_t*>(optr)[o] = static_cast<bf16_t>(acc[db][e] * oscale);
+        }
+      }
+    }
+  }
+}
+
+template <int MODE>
+int launch(const AttnBwdParams& bp, const float* lse2, hipStream_t st) {
+  auto kern = attn_bwd_dkdv_split_kernel<MODE>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) {
+      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      return MLTS_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  const int64_t blocks = static_cast<int64_t>(bp.nkt) * bp.a.B * bp.a.Hkv;
+  if (blocks > 0) {
+    MltsKernelTimer timer("attn_bwd_dkdv", st);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, bp, lse2);
+  }
+  return mlts_check_launch("mlts_attn_bwd");
+}
+
+}  // namespace
+
+// head_dim 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int mode, void* workspace, hipStream_t st) {
+  const AttnParams& p = bp.a;
+  bp.nkt = (p.Sk + BKV - 1) / BKV;
+  float* lse2 = static_cast<float*>(workspace);
+  const int64_t n = static_cast<int64_t>(p.B) * p.Hq * p.Sq;
+  hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 256) / 256)), dim3(256), 0, st, p.lse, lse2, n);
+  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(bp, lse2, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(bp, lse2, st);
+  return launch<MLTS_MASK_DOC>(bp, lse2, st);
+}
