@@ -1,0 +1,398 @@
+// Attention backward, dQ, head_dim 128, bf16: the version of attn_bwd_dq.hip with one LDS copy per tile.
+//
+// Same decomposition (a workgroup of 8 wavefronts owns 256 query rows of one (batch, head), each wavefront 32 of
+// them, Q and dO stay in registers, it walks the visible keys in tiles of 64 and recomputes the scores transposed so
+// that a lane owns one query and LSE / delta are per-lane scalars):
+//     S^T  = K Q^T             A = K rows (LDS)              B = Q  (registers)
+//     dlt - dP^T = dlt - V dO^T   A = V rows (LDS)              B = -dO (registers), accumulator starts at delta
+//     P = exp2(S c - lse2),  -dS = P (delta - dP)               registers; layout = B operand of the next product
+//     -dQ^T += K^T (-dS^T)     A = K^T (ds_read_b64_tr_b16 from the same K tile)
+// K and V tiles are fetched into registers right behind the barrier and written once, row major with the chunk
+// swizzle of attn_fwd_dma.hip, after the work on the current tile (two LDS stages); there is no transposed copy and
+// no VALU transposition.  LDS reads go through inline assembly with counted waits (see attn_fwd_dma.hip).
+#include "attn_common.hpp"
+#include <type_traits>
+
+namespace {
+
+constexpr int D = 128;
+constexpr int BN = 64;
+constexpr int WAVES = 8;
+constexpr int THREADS = WAVES * 64;
+constexpr int BM = WAVES * 32;
+constexpr int KS = D / 16;
+constexpr int DB = D / 32;
+constexpr int TILE_BYTES = BN * D * 2;       // 16 KiB
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K then V
+constexpr int STAGES = 2;
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+#define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+
+__device__ __forceinline__ void drain_and_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int OFF>
+__device__ __forceinline__ v4i32 lds_read_b128(uint32_t addr) {
+  v4i32 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ v2i32 lds_read_tr16_b64(uint32_t addr) {
+  v2i32 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write_b128(uint32_t addr, v4i32 x) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(x), "n"(OFF));
+}
+// wait_lgkm<N>(regs): only used when N or more LGKM operations of this code were issued after the reads into regs
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v2i32 (&x)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(%8)"
+               : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+               : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[2]) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x[0]), "+v"(x[1]) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v2i32 (&x)[4]) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : "n"(N));
+}
+__device__ __forceinline__ bf16x8 as_frag(v4i32 x) { return __builtin_bit_cast(bf16x8, x); }
+__device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+}
+
+template <int MODE>
+__global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdParams bp) {
+  const AttnParams& p = bp.a;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
+  const int nbh = p.B * p.Hq;
+  const int bid = blockIdx.x;
+  const int qt = p.nqt - 1 - bid / nbh;  // longest (last) q-tiles first under a causal mask
+  const int bh = bid % nbh;
+  const int b = bh / p.Hq, hq = bh % p.Hq;
+  const int hkv = hq / (p.Hq / p.Hkv);
+  const int q0 = qt * BM;
+  const int wq0 = q0 + wave * 32;
+  const int qrow = wq0 + l32;
+
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
+  const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1];
+  const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
+  const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
+
+  bf16x8 qf[KS], ndof[KS];  // Q and -dO fragments (B operands)
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    v4i32 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
+    if (qrow < p.Sq) {
+      a = *reinterpret_cast<const v4i32*>(Q + static_cast<int64_t>(qrow) * p.qs[2] + ks * 16 + hh * 8);
+      c = *reinterpret_cast<const v4i32*>(dO + static_cast<int64_t>(qrow) * bp.dos[2] + ks * 16 + hh * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c[i] ^= static_cast<int>(0x80008000u);
+    qf[ks] = as_frag(a);
+    ndof[ks] = as_frag(c);
+  }
+  float lse2 = INFINITY, delta = 0.f;  // +inf makes exp2(s - lse2) = 0 for rows that saw no key or lie past Sq
+  if (qrow < p.Sq) {
+    const int64_t off = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow;
+    const float l = p.lse[off];
+    lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
+    delta = bp.delta[off];
+  }
+  int qpos = 0, qseq = -1;
+  int4 wq_stats = make_int4(0, -1, 0, -1);
+  int4 bq_stats[BM / 64];
+  if (MODE == MLTS_MASK_DOC) {
+    if (qrow < p.Sq) {
+      qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qrow];
+      qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qrow];
+    }
+#pragma unroll
+    for (int w = 0; w < BM / 64; ++w) {
+      const int t = (q0 >> 6) + w;
+      bq_stats[w] = t < p.nq_stats ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
+    }
+    const int t = wq0 >> 6;
+    if (t < p.nq_stats) wq_stats = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t];
+  }
+
+  const int nkt = (p.Sk + BN - 1) / BN;
+  int j_end = nkt;
+  if (MODE == MLTS_MASK_CAUSAL) {
+    const int lim = min(q0 + BM, p.Sq) - 1 + p.causal_off;
+    j_end = lim < 0 ? 0 : min(nkt, lim / BN + 1);
+  }
+  const int wave_last_q = min(wq0 + 31, p.Sq - 1);
+  auto block_needs = [&](int j) -> bool {
+    if (MODE != MLTS_MASK_DOC) return true;
+    const int4 ks4 = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
+    bool need = false;
+#pragma unroll
+    for (int w = 0; w < BM / 64; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
+    return need;
+  };
+  auto next_tile = [&](int j) -> int {
+    while (j < j_end && !block_needs(j)) ++j;
+    return j;
+  };
+
+  // ---- tile loader: 64 bytes per thread, chunks t and t + 512 of the K tile and of the V tile (chunk c = row c/16,
+  // stored 16-byte slot c%16, source slot (c%16) ^ swz(row)); registers now, ds_write_b128 after this tile's work ----
+  int ld_row[2], ld_col[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int c = tid + n * THREADS;
+    ld_row[n] = c >> 4;
+    ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+  }
+  v4i32 stg_k[2], stg_v[2];
+  auto stage_load = [&](int j) {
+    const int kv0 = j * BN;
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
+      stg_k[n] = *reinterpret_cast<const v4i32*>(K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n]);
+      stg_v[n] = *reinterpret_cast<const v4i32*>(V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n]);
+    }
+  };
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
+  auto stage_store = [&](int stage) {
+    const uint32_t a = lds0 + stage * STAGE_BYTES + tid * 16;
+    lds_write_b128<0>(a, stg_k[0]);
+    lds_write_b128<THREADS * 16>(a, stg_k[1]);
+    lds_write_b128<TILE_BYTES>(a, stg_v[0]);
+    lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_v[1]);
+  };
+
+  // ---- per-lane LDS read offsets (tile invariant) ----
+  // (LDS addresses of stage 0; the stage, the key block and the tile are added as instruction offsets)
+  uint32_t ra[KS];  // row-major fragment (A operand): row l32 (+32 kb), chunk 2 ks + hh
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+  uint32_t ta[2][DB];  // K^T fragment halves: key row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4)
+#pragma unroll
+  for (int part = 0; part < 2; ++part) {
+    const int rlow = part * 8 + hh * 4 + (l16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
+      ta[part][db] = lds0 + rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+    }
+  }
+
+  f32x16 dqacc[DB];  // -dQ^T / scale: register e <-> head-dim 32 db + 8 (e/4) + 4 hh + e%4, lane -> query row
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dqacc[db][e] = 0.f;
+
+  // read groups are kept small (two 16-byte row reads, or four transpose reads) and two are in flight: the kernel
+  // sits at the 256-register limit of two wavefronts per SIMD
+#define MLTS_RREAD2(dst, KB, KS0)                                                  \
+  dst[0] = lds_read_b128<(KB) * 8192>(ra[(KS0)] + so);                             \
+  dst[1] = lds_read_b128<TILE_BYTES + (KB) * 8192>(ra[(KS0)] + so);
+#define MLTS_SMFMA2(src, KS0)                                                                            \
+  s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), qf[(KS0)], s, 0, 0, 0);                   \
+  dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), ndof[(KS0)], dp, 0, 0, 0);
+#define MLTS_TREAD4(dst, C, H)                                                       \
+  dst[0] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H)] + so);                       \
+  dst[1] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H)] + so);                       \
+  dst[2] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H) + 1] + so);                   \
+  dst[3] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H) + 1] + so);
+#define MLTS_TMFMA2(src, H, BFRAG)                                                                                        \
+  dqacc[2 * (H)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0], src[1]), BFRAG, dqacc[2 * (H)], 0, 0, 0);       \
+  dqacc[2 * (H) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2], src[3]), BFRAG, dqacc[2 * (H) + 1], 0, 0, 0);
+
+  // one 64-key tile for this wavefront's 32 queries, one 32-key block after the other; lane = query, accumulator
+  // register e <-> key 32 kb + 8 (e/4) + 4 hh + e%4
+  auto process_tile = [&](auto masked_tag, const uint32_t so, const int kv0) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const int klim_t = min(qrow + (MODE == MLTS_MASK_CAUSAL ? p.causal_off : 0x3fffffff), p.Sk - 1) - kv0 - hh * 4;
+    bf16x8 dsf[2];
+    f32x16 s, dp;
+    auto ds_block = [&](const int kb) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+        int kp[4], ksq[4];
+        if (MASKED && MODE == MLTS_MASK_DOC) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int kj = kbase + r;
+            const bool ok = kj < p.Sk;
+            kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
+            ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int e = g * 4 + r;
+          float pv = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse2);
+          if (MASKED) {
+            // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
+            bool vis = kb * 32 + g * 8 + r <= klim_t;
+            if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+            if (!vis) pv = 0.f;
+          }
+          dsf[e >> 3][e & 7] = static_cast<bf16_t>(pv * dp[e]);  // -dS
+        }
+      }
+    };
+    auto acc_init = [&]() {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        s[e] = 0.f;
+        dp[e] = delta;
+      }
+    };
+    v4i32 g0[2], g1[2];
+    v2i32 h0[4], h1[4];
+#define MLTS_KEY_BLOCK(KB)                                                         \
+    acc_init();                                                                    \
+    MLTS_RREAD2(g0, KB, 0)                                                         \
+    MLTS_RREAD2(g1, KB, 1)                                                         \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 0) MLTS_RREAD2(g0, KB, 2)                    \
+    wait_lgkm<2>(g1); MLTS_SMFMA2(g1, 1) MLTS_RREAD2(g1, KB, 3)                    \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 2) MLTS_RREAD2(g0, KB, 4)                    \
+    wait_lgkm<2>(g1); MLTS_SMFMA2(g1, 3) MLTS_RREAD2(g1, KB, 5)                    \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 4) MLTS_RREAD2(g0, KB, 6)                    \
+    wait_lgkm<2>(g1); MLTS_SMFMA2(g1, 5) MLTS_RREAD2(g1, KB, 7)                    \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 6) MLTS_TREAD4(h0, 2 * (KB), 0)              \
+    wait_lgkm<4>(g1); MLTS_SMFMA2(g1, 7) MLTS_TREAD4(h1, 2 * (KB), 1)              \
+    ds_block(KB);                                                                  \
+    wait_lgkm<4>(h0); MLTS_TMFMA2(h0, 0, dsf[0]) MLTS_TREAD4(h0, 2 * (KB) + 1, 0)  \
+    wait_lgkm<4>(h1); MLTS_TMFMA2(h1, 1, dsf[0]) MLTS_TREAD4(h1, 2 * (KB) + 1, 1)  \
+    wait_lgkm<4>(h0); MLTS_TMFMA2(h0, 0, dsf[1])                                   \
+    wait_lgkm<0>(h1); MLTS_TMFMA2(h1, 1, dsf[1])
+    MLTS_KEY_BLOCK(0)
+    MLTS_KEY_BLOCK(1)
+#undef MLTS_KEY_BLOCK
+  };
+#undef MLTS_RREAD2
+#undef MLTS_SMFMA2
+#undef MLTS_TREAD4
+#undef MLTS_TMFMA2
+
+  // ---- tile loop.  Barrier k: tile k is in LDS.  Tile k + 1 is fetched behind it into registers and stored into the
+  // other stage (read last during tile k - 1) after the work on tile k.  POLICY: 0 = no tile needs masking, 1 = every
+  // tile is masked (the comparison costs two VALU operations per score), 2 = by tile class.  One instance of the tile
+  // body per loop where possible: with several, the register allocator keeps the dQ accumulators twice. ----
+  auto tile_loop = [&](auto policy_tag) {
+    constexpr int POLICY = decltype(policy_tag)::value;
+    int j = next_tile(0);
+    if (j < j_end) {
+      stage_load(j);
+      stage_store(0);
+    }
+    int stage = 0;
+    while (j < j_end) {
+      const int jn = next_tile(j + 1);
+      drain_and_barrier();
+      if (jn < j_end) stage_load(jn);
+
+      const int kv0 = j * BN;
+      int cls = TILE_FULL;
+      if (MODE == MLTS_MASK_CAUSAL) {
+        if (kv0 > wave_last_q + p.causal_off) cls = TILE_SKIP;
+      } else if (MODE == MLTS_MASK_DOC) {
+        cls = classify_doc_tile(wq_stats, p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j]);
+        if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;
+      }
+      if (wq0 >= p.Sq) cls = TILE_SKIP;
+      const uint32_t so = stage * STAGE_BYTES;
+      if (POLICY == 0) {
+        if (cls != TILE_SKIP) process_tile(std::false_type{}, so, kv0);
+      } else if (POLICY == 1) {
+        if (cls != TILE_SKIP) process_tile(std::true_type{}, so, kv0);
+      } else {
+        if (cls == TILE_FULL) process_tile(std::false_type{}, so, kv0);
+        else if (cls == TILE_MASKED) process_tile(std::true_type{}, so, kv0);
+      }
+
+      if (jn < j_end) stage_store(stage ^ 1);
+      j = jn;
+      stage ^= 1;
+    }
+  };
+  if (MODE == MLTS_MASK_CAUSAL) {
+    tile_loop(std::integral_constant<int, 1>{});
+  } else if (MODE == MLTS_MASK_DOC) {
+    tile_loop(std::integral_constant<int, 2>{});
+  } else if (p.Sk % BN != 0) {
+    tile_loop(std::integral_constant<int, 1>{});  // the ragged last tile needs key < Sk
+  } else {
+    tile_loop(std::integral_constant<int, 0>{});
+  }
+
+  if (qrow < p.Sq) {
+    const float oscale = -p.scale;  // the accumulator holds K^T (-dS^T)
+    const int64_t rowoff = b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(qrow) * bp.dqs[2];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8 + hh * 4;
+        if (bp.accumulate_f32) {
+          f32x4* dst = reinterpret_cast<f32x4*>(bp.dq_acc + rowoff + d);
+          f32x4 cur = *dst;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) cur[r] += dqacc[db][g * 4 + r] * oscale;
+          *dst = cur;
+        } else {
+          bf16x4 w;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(dqacc[db][g * 4 + r] * oscale);
+          *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(bp.dq_acc) + rowoff + d) = w;
+        }
+      }
+    }
+  }
+}
+
+template <int MODE>
+int launch(AttnBwdParams bp, hipStream_t st) {
+  auto kern = attn_bwd_dq_tr_kernel<MODE>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) {
+      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      return MLTS_ERR_LAUNCH;
+    }
+    configured = true;
+  }
+  bp.a.nqt = (bp.a.Sq + BM - 1) / BM;
+  const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * bp.a.Hq;
+  if (blocks > 0) {
+    MltsKernelTimer timer("attn_bwd_dq", st);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, bp);
+  }
+  return mlts_check_launch("mlts_attn_bwd");
+}
+
+}  // namespace
+
+// head_dim 128, Sk >= 1 when Sq >= 1 reaches a key, 16-byte aligned rows (checked by the caller)
+int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int mode, hipStream_t st) {
+  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(bp, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(bp, st);
+  return launch<MLTS_MASK_DOC>(bp, st);
+}

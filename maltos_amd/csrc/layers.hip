@@ -137,19 +137,38 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restri
   }
 }
 
+// dw[col] = sum over the per-block partial rows, in a fixed order: a block owns 32 columns, its 8 groups of 32
+// lanes each add every 8th partial row (four loads in flight), then the 8 group sums are added through LDS.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void rmsnorm_dw_reduce_kernel(const float* __restrict__ dw_partial, int nblocks,
                                                                      int hidden, T* __restrict__ dw) {
-  const int col = blockIdx.x * kThreads + threadIdx.x;
-  if (col >= hidden) return;
-  float s = 0.f;
-  for (int b = 0; b < nblocks; ++b) s += dw_partial[static_cast<int64_t>(b) * hidden + col];
-  dw[col] = from_f32<T>(s);
+  __shared__ float part[8][32];
+  const int c = threadIdx.x & 31, r = threadIdx.x >> 5;
+  const int col = blockIdx.x * 32 + c;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (col < hidden) {
+    int b = r;
+    for (; b + 24 < nblocks; b += 32) {
+      s0 += dw_partial[static_cast<int64_t>(b) * hidden + col];
+      s1 += dw_partial[static_cast<int64_t>(b + 8) * hidden + col];
+      s2 += dw_partial[static_cast<int64_t>(b + 16) * hidden + col];
+      s3 += dw_partial[static_cast<int64_t>(b + 24) * hidden + col];
+    }
+    for (; b < nblocks; b += 8) s0 += dw_partial[static_cast<int64_t>(b) * hidden + col];
+  }
+  part[r][c] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (r == 0 && col < hidden) {
+    float s = part[0][c];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) s += part[i][c];
+    dw[col] = from_f32<T>(s);
+  }
 }
 
 int rmsnorm_bwd_blocks(int64_t rows) {
   int64_t b = (rows + 31) / 32;  // >= 32 rows per block keeps the partial buffer small
-  if (b > 1024) b = 1024;
+  if (b > 256) b = 256;          // one block per CU; more only lengthens the reduction above
   if (b < 1) b = 1;
   return static_cast<int>(b);
 }
@@ -293,7 +312,7 @@ int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rst
   hipLaunchKernelGGL(rmsnorm_bwd_kernel<T>, dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy),
                      static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,
                      hidden, rows_per_block);
-  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + kThreads - 1) / kThreads), dim3(kThreads), 0, st,
+  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + 31) / 32), dim3(kThreads), 0, st,
                      partial, blocks, hidden, static_cast<T*>(dw));
   return mlts_check_launch("mlts_rmsnorm_bwd");
 }
