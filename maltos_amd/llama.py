@@ -41,6 +41,52 @@ class LlamaConfig:
         validate_attention_backend(self.attention_backend)
 
 
+def _weight_grad_splits(rows: int, out_features: int, in_features: int) -> int:
+    """Number of K-splits for dW = dY^T X.  The product has only out*in outputs but `rows` (= tokens) terms each:
+    for the LLaMA-50M projections (512..1536 wide, 16384 tokens) a single GEMM fills a quarter of the 256 CUs and
+    runs at ~85 TFLOP/s, the same work as a batch of 8-16 row slices reaches 300-600 TFLOP/s on MI355X."""
+    tiles = -(-out_features // 256) * -(-in_features // 256)
+    splits = 1
+    while splits < 16 and tiles * splits < 128 and rows % (splits * 2) == 0 and rows // (splits * 2) >= 1024:
+        splits *= 2
+    return splits
+
+
+class _SplitKLinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        ctx.save_for_backward(x, weight)
+        return F.linear(x, weight)
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        x, weight = ctx.saved_tensors
+        dx = dw = None
+        if ctx.needs_input_grad[0]:
+            dx = dy.matmul(weight)
+        if ctx.needs_input_grad[1]:
+            x2 = x.reshape(-1, x.shape[-1])
+            dy2 = dy.reshape(-1, dy.shape[-1])
+            splits = _weight_grad_splits(x2.shape[0], dy2.shape[1], x2.shape[1])
+            if splits > 1 and x2.is_contiguous() and dy2.is_contiguous():
+                rows = x2.shape[0] // splits
+                part = torch.bmm(dy2.view(splits, rows, -1).transpose(1, 2), x2.view(splits, rows, -1))
+                dw = part.sum(0, dtype=torch.float32).to(weight.dtype)  # slices added in fp32, rounded once
+            else:
+                dw = dy2.t().matmul(x2)
+        return dx, dw
+
+
+class HipLinear(nn.Linear):
+    """nn.Linear (same parameter name and init) whose weight gradient is computed as a batch of row slices when the
+    output is too small to fill the chip (reference: plain nn.Linear, models/llama.py:69-75,196-198)."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.bias is not None or not x.is_cuda:
+            return F.linear(x, self.weight, self.bias)
+        return _SplitKLinearFn.apply(x, self.weight)
+
+
 class LlamaRMSNorm(nn.Module):
     def __init__(self, hidden_size: int, eps: float) -> None:
         super().__init__()
@@ -99,10 +145,10 @@ class LlamaAttention(nn.Module):
             raise ValueError("num_attention_heads must be divisible by num_key_value_heads")
         self.head_dim = config.hidden_size // config.num_attention_heads
         self.rotary_emb = LlamaRotaryEmbedding(self.head_dim, config.max_position_embeddings, config.rope_theta)
-        self.q_proj = nn.Linear(config.hidden_size, self.num_heads * self.head_dim, bias=False)
-        self.k_proj = nn.Linear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
-        self.v_proj = nn.Linear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
-        self.o_proj = nn.Linear(config.hidden_size, config.hidden_size, bias=False)
+        self.q_proj = HipLinear(config.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = HipLinear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.v_proj = HipLinear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.o_proj = HipLinear(config.hidden_size, config.hidden_size, bias=False)
         self.attn_core = HipAttentionCore(config.attention_backend)
 
     def forward(self, x: torch.Tensor, *, position_offset: int = 0, position_ids: torch.Tensor | None = None,
@@ -129,9 +175,9 @@ class LlamaAttention(nn.Module):
 class LlamaMLP(nn.Module):
     def __init__(self, config: LlamaConfig) -> None:
         super().__init__()
-        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
-        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
-        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+        self.gate_proj = HipLinear(config.hidden_size, config.intermediate_size, bias=False)
+        self.up_proj = HipLinear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = HipLinear(config.intermediate_size, config.hidden_size, bias=False)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.down_proj(ops.swiglu(self.gate_proj(x), self.up_proj(x)))
