@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled
 # by the same counters over the --calibrate-traffic kernel (summary: profiles/attn_cfg2_hbm_traffic.md).  Counters
 # cannot be read from inside the timed run, so the figures are carried here and refreshed with the profile.
-MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 619.0e6, "attn_bwd_dkdv": 885.3e6, "attn_bwd_dq": 841.4e6}
+MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 612.0e6, "attn_bwd_dkdv": 885.8e6, "attn_bwd_dq": 651.3e6}
 
 
 def parse_args():
