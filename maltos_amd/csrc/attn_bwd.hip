@@ -422,9 +422,13 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   int rc;
-  if (dkdv_variant(D) == 2) {
+  int variant = dkdv_variant(D);
+  // the newer kernels address rows of a tile with 32-bit element offsets
+  const int64_t lim = int64_t{1} << 24;
+  if (p.qs[2] >= lim || p.ks[2] >= lim || p.vs[2] >= lim || bp.dos[2] >= lim) variant = 0;
+  if (variant == 2) {
     rc = mlts_attn_bwd_dkdv_bf16_split(bp, mode, workspace, st);
-  } else if (dkdv_variant(D) == 1) {
+  } else if (variant == 1) {
     rc = mlts_attn_bwd_dkdv_bf16_dma(bp, mode, workspace, st);
   } else if (D == 128) {
     if (mode == MLTS_MASK_NONE) rc = launch_bwd<128, MLTS_MASK_NONE>(bp, st);
@@ -436,6 +440,6 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
-  if (dkdv_variant(D) == 2) return mlts_attn_bwd_dq_bf16_tr(bp, mode, st);
+  if (variant == 2) return mlts_attn_bwd_dq_bf16_tr(bp, mode, st);
   return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

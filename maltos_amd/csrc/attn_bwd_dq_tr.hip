@@ -156,21 +156,34 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   // ---- tile loader: 64 bytes per thread, chunks t and t + 512 of the K tile and of the V tile (chunk c = row c/16,
   // stored 16-byte slot c%16, source slot (c%16) ^ swz(row)); registers now, ds_write_b128 after this tile's work ----
+  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
+  // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
   int ld_row[2], ld_col[2];
+  uint32_t ld_koff[2], ld_voff[2];
 #pragma unroll
   for (int n = 0; n < 2; ++n) {
     const int c = tid + n * THREADS;
     ld_row[n] = c >> 4;
     ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+    ld_koff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.ks[2]) + ld_col[n];
+    ld_voff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n];
   }
   v4i32 stg_k[2], stg_v[2];
   auto stage_load = [&](int j) {
     const int kv0 = j * BN;
+    const bf16_t* Kt = K + static_cast<int64_t>(kv0) * p.ks[2];
+    const bf16_t* Vt = V + static_cast<int64_t>(kv0) * p.vs[2];
+    const int last = p.Sk - 1 - kv0;  // rows past the end repeat the last key; their scores are masked
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
-      const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
-      stg_k[n] = *reinterpret_cast<const v4i32*>(K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n]);
-      stg_v[n] = *reinterpret_cast<const v4i32*>(V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n]);
+      uint32_t ko = ld_koff[n], vo = ld_voff[n];
+      if (last < BN - 1) {
+        const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
+        ko = r * static_cast<uint32_t>(p.ks[2]) + ld_col[n];
+        vo = r * static_cast<uint32_t>(p.vs[2]) + ld_col[n];
+      }
+      stg_k[n] = *reinterpret_cast<const v4i32*>(Kt + ko);
+      stg_v[n] = *reinterpret_cast<const v4i32*>(Vt + vo);
     }
   };
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));

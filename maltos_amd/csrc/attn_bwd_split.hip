@@ -5,6 +5,7 @@
 // block kb = wave % 4:
 //     role 0 (wave < 4):   S = Q K^T,  P = exp2(S c - lse2)  ->  dV += P^T dO      and hands P (bf16) over in LDS
 //     role 1 (wave >= 4):  delta - dO V^T,  -dS = P (delta - dO V^T)  ->  -dK += (-dS)^T Q     one tile behind
+//                          (per barrier interval: dS of tile k-1, dP of tile k, then the dK products of tile k-1)
 // Each role keeps one operand (K or -V) and one accumulator (dV or dK) in registers, so a wavefront fits in
 // 256 registers, two wavefronts share a SIMD, the matrix instructions take plain VGPR accumulators (no AGPR
 // copies around the softmax arithmetic) and the hardware overlaps one wavefront's VALU work with the other's
@@ -189,12 +190,17 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   // source slot (c%16) ^ swz(row)) and written to LDS with ds_write_b128 after this tile's work.  Threads 0..127 also
   // carry the 64 + 64 row statistics (lse2, delta). ----
   const int64_t lse2_inf = static_cast<int64_t>(p.B) * p.Hq * p.Sq;  // index of the +inf entry
+  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
+  // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
   int ld_row[2], ld_col[2];
+  uint32_t ld_qoff[2], ld_doff[2];
 #pragma unroll
   for (int n = 0; n < 2; ++n) {
     const int c = tid + n * THREADS;
     ld_row[n] = c >> 4;
     ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+    ld_qoff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.qs[2]) + ld_col[n];
+    ld_doff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(bp.dos[2]) + ld_col[n];
   }
   v4i32 stg_q[2], stg_d[2];
   float stg_s = 0.f;
@@ -202,13 +208,19 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   auto stage_load = [&](int it) {
     const int hq = hkv * group + it / span;
     const int q0 = (qt_begin + it % span) * BQ;
-    const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
-    const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1];
+    const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1] + static_cast<int64_t>(q0) * p.qs[2];
+    const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1] + static_cast<int64_t>(q0) * bp.dos[2];
+    const int last = p.Sq - 1 - q0;  // rows past the end repeat the last query; their lse2 is +inf
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
-      const int r = min(q0 + ld_row[n], p.Sq - 1);  // rows past the end repeat the last query; their lse2 is +inf
-      stg_q[n] = *reinterpret_cast<const v4i32*>(Q + static_cast<int64_t>(r) * p.qs[2] + ld_col[n]);
-      stg_d[n] = *reinterpret_cast<const v4i32*>(dO + static_cast<int64_t>(r) * bp.dos[2] + ld_col[n]);
+      uint32_t qo = ld_qoff[n], dofs = ld_doff[n];
+      if (last < BQ - 1) {
+        const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
+        qo = r * static_cast<uint32_t>(p.qs[2]) + ld_col[n];
+        dofs = r * static_cast<uint32_t>(bp.dos[2]) + ld_col[n];
+      }
+      stg_q[n] = *reinterpret_cast<const v4i32*>(Q + qo);
+      stg_d[n] = *reinterpret_cast<const v4i32*>(dO + dofs);
     }
     if (tid < 2 * BQ) {
       const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
@@ -413,24 +425,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     wait_lgkm<0>(g1);
     MLTS_RMFMA4(g1, dp1, 4)
   };
-  // ---- role 1, second half (one barrier later): -dS = P dp, -dK += (-dS)^T Q ----
-  auto role1_dk = [&](const int stage, const int pbuf) {
-    const uint32_t sb = lds0 + stage * STAGE_BYTES;
-    uint32_t ta[2][DB];
-#pragma unroll
-    for (int part = 0; part < 2; ++part)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+  // ---- role 1, one barrier later: -dS = P dp as soon as P has arrived (frees dp for the next tile) ... ----
+  bf16x8 dsfr[4];
+  auto role1_ds = [&](const int pbuf) {
     v4i32 pp[4];
-    v2i32 h0[8], h1[8];
     pp[0] = lds_read_b128<0>(pbuf_lane + pbuf);
     pp[1] = lds_read_b128<1024>(pbuf_lane + pbuf);
     pp[2] = lds_read_b128<2048>(pbuf_lane + pbuf);
     pp[3] = lds_read_b128<3072>(pbuf_lane + pbuf);
-    MLTS_TREAD8(h0, 0)
-    MLTS_TREAD8(h1, 1)
-    wait_lgkm<15>(pp);  // 16 reads follow; the counter field holds at most 15
-    bf16x8 dsfr[4];
+    wait_lgkm<0>(pp);
 #pragma unroll
     for (int f = 0; f < 4; ++f) {
 #pragma unroll
@@ -444,6 +447,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         dsfr[f][2 * w + 1] = static_cast<bf16_t>(phi * dhi);
       }
     }
+  };
+  // ---- ... and, after the dp of the next tile, -dK += (-dS)^T Q (transposed reads, while role 0 does its softmax) ----
+  auto role1_dk = [&](const int stage) {
+    const uint32_t sb = lds0 + stage * STAGE_BYTES;
+    uint32_t ta[2][DB];
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+    v2i32 h0[8], h1[8];
+    MLTS_TREAD8(h0, 0)
+    MLTS_TREAD8(h1, 1)
     wait_lgkm<8>(h0);
     MLTS_TMFMA4(h0, dsfr[0])
     MLTS_TREAD8(h0, 2)
@@ -493,8 +508,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
           else if (cls == TILE_MASKED) role0_tile(std::true_type{}, q0, stage, pbuf);
         }
       } else {
-        if (prev_active) role1_dk(prev_stage, pbuf ^ (4 * PBUF_BYTES));
+        if (prev_active) role1_ds(pbuf ^ (4 * PBUF_BYTES));
         if (cls != TILE_SKIP) role1_dp(stage);
+        if (prev_active) role1_dk(prev_stage);
       }
       if (itn < total_it) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
       prev_active = cls != TILE_SKIP;
@@ -504,7 +520,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       ++k;
     }
     drain_and_barrier();
-    if (ROLE == 1 && prev_active) role1_dk(prev_stage, ((k - 1) & 1) * (4 * PBUF_BYTES));
+    if (ROLE == 1 && prev_active) {
+      role1_ds(((k - 1) & 1) * (4 * PBUF_BYTES));
+      role1_dk(prev_stage);
+    }
   };
   if (role == 0) tile_loop(std::integral_constant<int, 0>{});
   else tile_loop(std::integral_constant<int, 1>{});
