@@ -236,17 +236,17 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   // one 64-key tile for this wavefront's 32 queries, one 32-key block after the other; lane = query, accumulator
   // register e <-> key 32 kb + 8 (e/4) + 4 hh + e%4
-  auto process_tile = [&](auto masked_tag, const uint32_t so, const int kv0) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
+  auto process_tile = [&](const bool masked, const uint32_t so, const int kv0) {
     const int klim_t = min(qrow + (MODE == MLTS_MASK_CAUSAL ? p.causal_off : 0x3fffffff), p.Sk - 1) - kv0 - hh * 4;
     bf16x8 dsf[2];
     f32x16 s, dp;
-    auto ds_block = [&](const int kb) {
+    // masked tiles only (a wave-uniform branch around VALU work, no matrix instruction inside): hidden scores -> -inf
+    auto apply_mask = [&](const int kb) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
         int kp[4], ksq[4];
-        if (MASKED && MODE == MLTS_MASK_DOC) {
+        if (MODE == MLTS_MASK_DOC) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int kj = kbase + r;
@@ -257,16 +257,27 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int e = g * 4 + r;
-          float pv = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse2);
-          if (MASKED) {
-            // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
-            bool vis = kb * 32 + g * 8 + r <= klim_t;
-            if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
-            if (!vis) pv = 0.f;
-          }
-          dsf[e >> 3][e & 7] = static_cast<bf16_t>(pv * dp[e]);  // -dS
+          // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
+          bool vis = kb * 32 + g * 8 + r <= klim_t;
+          if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+          if (!vis) s[g * 4 + r] = -INFINITY;
         }
+      }
+    };
+    auto ds_block = [&](const int kb) {
+      if (masked) apply_mask(kb);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        v4i32 w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // elements 8 t + 2 j, + 1 -> one packed conversion of -dS
+          const int e = t * 8 + 2 * j;
+          f32x2 ds;
+          ds[0] = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse2) * dp[e];
+          ds[1] = __builtin_amdgcn_exp2f(s[e + 1] * p.scale_log2 - lse2) * dp[e + 1];
+          w[j] = __builtin_bit_cast(int, __builtin_convertvector(ds, bf16x2));
+        }
+        dsf[t] = __builtin_bit_cast(bf16x8, w);
       }
     };
     auto acc_init = [&]() {
@@ -305,11 +316,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #undef MLTS_TMFMA2
 
   // ---- tile loop.  Barrier k: tile k is in LDS.  Tile k + 1 is fetched behind it into registers and stored into the
-  // other stage (read last during tile k - 1) after the work on tile k.  POLICY: 0 = no tile needs masking, 1 = every
-  // tile is masked (the comparison costs two VALU operations per score), 2 = by tile class.  One instance of the tile
-  // body per loop where possible: with several, the register allocator keeps the dQ accumulators twice. ----
-  auto tile_loop = [&](auto policy_tag) {
-    constexpr int POLICY = decltype(policy_tag)::value;
+  // other stage (read last during tile k - 1) after the work on tile k.  There is one instance of the tile body
+  // (with several, the register allocator keeps the dQ accumulators twice); masking is a branch inside it. ----
+  {
     int j = next_tile(0);
     if (j < j_end) {
       stage_load(j);
@@ -325,34 +334,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       int cls = TILE_FULL;
       if (MODE == MLTS_MASK_CAUSAL) {
         if (kv0 > wave_last_q + p.causal_off) cls = TILE_SKIP;
+        else if (kv0 + BN - 1 > wq0 + p.causal_off) cls = TILE_MASKED;
       } else if (MODE == MLTS_MASK_DOC) {
         cls = classify_doc_tile(wq_stats, p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j]);
-        if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;
       }
+      if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;  // ragged last tile: key < Sk
       if (wq0 >= p.Sq) cls = TILE_SKIP;
-      const uint32_t so = stage * STAGE_BYTES;
-      if (POLICY == 0) {
-        if (cls != TILE_SKIP) process_tile(std::false_type{}, so, kv0);
-      } else if (POLICY == 1) {
-        if (cls != TILE_SKIP) process_tile(std::true_type{}, so, kv0);
-      } else {
-        if (cls == TILE_FULL) process_tile(std::false_type{}, so, kv0);
-        else if (cls == TILE_MASKED) process_tile(std::true_type{}, so, kv0);
-      }
+      if (cls != TILE_SKIP) process_tile(cls == TILE_MASKED, stage * STAGE_BYTES, kv0);
 
       if (jn < j_end) stage_store(stage ^ 1);
       j = jn;
       stage ^= 1;
     }
-  };
-  if (MODE == MLTS_MASK_CAUSAL) {
-    tile_loop(std::integral_constant<int, 1>{});
-  } else if (MODE == MLTS_MASK_DOC) {
-    tile_loop(std::integral_constant<int, 2>{});
-  } else if (p.Sk % BN != 0) {
-    tile_loop(std::integral_constant<int, 1>{});  // the ragged last tile needs key < Sk
-  } else {
-    tile_loop(std::integral_constant<int, 0>{});
   }
 
   if (qrow < p.Sq) {

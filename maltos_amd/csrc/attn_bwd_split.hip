@@ -284,8 +284,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       __builtin_amdgcn_mfma_f32_32x32x16_bf16(AFRAG, as_frag(src[2 * db], src[2 * db + 1]), acc[db], 0, 0, 0);
 
   // ---- role 0: one tile.  lane = key, accumulator register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4 ----
-  auto role0_tile = [&](auto masked_tag, const int q0, const int stage, const int pbuf) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
+  auto role0_tile = [&](const bool masked, const int q0, const int stage, const int pbuf) {
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
     uint32_t ra[KS];
 #pragma unroll
@@ -299,13 +298,14 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     const int causal_t = kj - p.causal_off - q0 - hh * 4;
 
     bf16x8 pfr[2][2];
-    auto softmax = [&](auto qb_tag, const f32x16& s, const f32x4 (&lse4)[4]) {
+    // masked tiles only (a wave-uniform branch around VALU work, no matrix instruction inside): hidden scores -> -inf
+    auto apply_mask = [&](auto qb_tag, f32x16& s) {
       constexpr int qb = decltype(qb_tag)::value;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int qrow = qb * 32 + g * 8 + hh * 4;
         int qp4[4], qs4[4];
-        if (MASKED && MODE == MLTS_MASK_DOC) {
+        if (MODE == MLTS_MASK_DOC) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int qi = q0 + qrow + r;
@@ -316,20 +316,31 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int e = g * 4 + r;
-          float pv = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse4[g][r]);
-          if (MASKED) {
-            bool vis;
-            if (MODE == MLTS_MASK_CAUSAL) {
-              vis = causal_t <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
-            } else {
-              const int qi = q0 + qrow + r;
-              vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
-            }
-            if (!vis) pv = 0.f;
+          bool vis;
+          if (MODE == MLTS_MASK_CAUSAL) {
+            vis = causal_t <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
+          } else {
+            const int qi = q0 + qrow + r;
+            vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
           }
-          pfr[qb][e >> 3][e & 7] = static_cast<bf16_t>(pv);
+          if (!vis) s[g * 4 + r] = -INFINITY;
         }
+      }
+    };
+    auto softmax = [&](auto qb_tag, const f32x16& s, const f32x4 (&lse4)[4]) {
+      constexpr int qb = decltype(qb_tag)::value;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        v4i32 w;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // elements 8 t + 2 j, + 1 -> one packed conversion
+          const int e = t * 8 + 2 * j;
+          f32x2 pv;
+          pv[0] = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse4[e >> 2][e & 3]);
+          pv[1] = __builtin_amdgcn_exp2f(s[e + 1] * p.scale_log2 - lse4[(e + 1) >> 2][(e + 1) & 3]);
+          w[j] = __builtin_bit_cast(int, __builtin_convertvector(pv, bf16x2));
+        }
+        pfr[qb][t] = __builtin_bit_cast(bf16x8, w);
       }
     };
     using I0 = std::integral_constant<int, 0>;
@@ -364,6 +375,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     // whole-vector casts: casting a single element of an asm result is miscompiled (element 0 is broadcast)
 #pragma unroll
     for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
+    if (masked) apply_mask(I0{}, s0);
     softmax(I0{}, s0, lse4);
     wait_lgkm<8>(g1);
     MLTS_RMFMA4(g1, s1, 4)
@@ -375,6 +387,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     MLTS_TREAD8(h0, 2)
 #pragma unroll
     for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
+    if (masked) apply_mask(I1{}, s1);
     softmax(I1{}, s1, lse4);
     wait_lgkm<8>(h1);
     MLTS_TMFMA4(h1, pfr[0][1])
@@ -496,17 +509,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       const int cls = classify(it);
       const int pbuf = (k & 1) * (4 * PBUF_BYTES);
       if (ROLE == 0) {
-        // one instance of the tile body per mask mode where possible: without a mask nothing needs masking (keys
-        // past Sk are never stored, queries past Sq have lse2 = +inf), the causal comparison is cheap enough to be
-        // always on
-        if (MODE == MLTS_MASK_NONE) {
-          if (cls != TILE_SKIP) role0_tile(std::false_type{}, q0, stage, pbuf);
-        } else if (MODE == MLTS_MASK_CAUSAL) {
-          if (cls != TILE_SKIP) role0_tile(std::true_type{}, q0, stage, pbuf);
-        } else {
-          if (cls == TILE_FULL) role0_tile(std::false_type{}, q0, stage, pbuf);
-          else if (cls == TILE_MASKED) role0_tile(std::true_type{}, q0, stage, pbuf);
-        }
+        // one instance of the tile body (with several, the register allocator keeps the accumulators twice); the
+        // mask is a branch around VALU work inside it.  Without a mask mode nothing needs masking: keys past Sk are
+        // never stored and queries past Sq have lse2 = +inf.
+        if (cls != TILE_SKIP) role0_tile(MODE != MLTS_MASK_NONE && cls == TILE_MASKED, q0, stage, pbuf);
       } else {
         if (prev_active) role1_ds(pbuf ^ (4 * PBUF_BYTES));
         if (cls != TILE_SKIP) role1_dp(stage);
