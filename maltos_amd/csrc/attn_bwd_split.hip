@@ -327,22 +327,33 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         }
       }
     };
-    auto softmax = [&](auto qb_tag, const f32x16& s, const f32x4 (&lse4)[4]) {
+    // one P fragment (8 of the 16 scores of a query block): exp2, packed conversion
+    auto softmax_half = [&](auto qb_tag, auto t_tag, const f32x16& s, const f32x4 (&lse4)[4]) {
       constexpr int qb = decltype(qb_tag)::value;
+      constexpr int t = decltype(t_tag)::value;
+      v4i32 w;
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        v4i32 w;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {  // elements 8 t + 2 j, + 1 -> one packed conversion
-          const int e = t * 8 + 2 * j;
-          f32x2 pv;
-          pv[0] = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse4[e >> 2][e & 3]);
-          pv[1] = __builtin_amdgcn_exp2f(s[e + 1] * p.scale_log2 - lse4[(e + 1) >> 2][(e + 1) & 3]);
-          w[j] = __builtin_bit_cast(int, __builtin_convertvector(pv, bf16x2));
-        }
-        pfr[qb][t] = __builtin_bit_cast(bf16x8, w);
+      for (int j = 0; j < 4; ++j) {  // elements 8 t + 2 j, + 1 -> one packed conversion
+        const int e = t * 8 + 2 * j;
+        f32x2 pv;
+        pv[0] = __builtin_amdgcn_exp2f(s[e] * p.scale_log2 - lse4[e >> 2][e & 3]);
+        pv[1] = __builtin_amdgcn_exp2f(s[e + 1] * p.scale_log2 - lse4[(e + 1) >> 2][(e + 1) & 3]);
+        w[j] = __builtin_bit_cast(int, __builtin_convertvector(pv, bf16x2));
       }
+      pfr[qb][t] = __builtin_bit_cast(bf16x8, w);
     };
+    // A wavefront can issue one MFMA per 32 cycles and VALU work in between: the four MFMAs of a group are spread
+    // through the ~20 VALU instructions of half a softmax instead of being issued back to back.
+#define MLTS_INTERLEAVE_4MFMA(NV)                                   \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+  __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);               \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+  __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);               \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+  __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);               \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+  __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);               \
+  __builtin_amdgcn_sched_barrier(0);
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
 
@@ -369,28 +380,38 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     MLTS_RMFMA4(g1, s0, 4)
     MLTS_RREAD4(g1, 1, 4)
     wait_lgkm<8>(st1);
-    wait_lgkm<4>(g0);
-    MLTS_RMFMA4(g0, s1, 0)
-    MLTS_TREAD8(h0, 0)
     // whole-vector casts: casting a single element of an asm result is miscompiled (element 0 is broadcast)
 #pragma unroll
     for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
     if (masked) apply_mask(I0{}, s0);
-    softmax(I0{}, s0, lse4);
+    wait_lgkm<4>(g0);
+    __builtin_amdgcn_sched_barrier(0);
+    MLTS_RMFMA4(g0, s1, 0)
+    softmax_half(I0{}, I0{}, s0, lse4);
+    MLTS_INTERLEAVE_4MFMA(5)
+    MLTS_TREAD8(h0, 0)
     wait_lgkm<8>(g1);
+    __builtin_amdgcn_sched_barrier(0);
     MLTS_RMFMA4(g1, s1, 4)
+    softmax_half(I0{}, I1{}, s0, lse4);
+    MLTS_INTERLEAVE_4MFMA(5)
     MLTS_TREAD8(h1, 1)
     lds_write_b128<0>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][0]));
     lds_write_b128<1024>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][1]));
-    wait_lgkm<10>(h0);
-    MLTS_TMFMA4(h0, pfr[0][0])
-    MLTS_TREAD8(h0, 2)
 #pragma unroll
     for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
     if (masked) apply_mask(I1{}, s1);
-    softmax(I1{}, s1, lse4);
+    wait_lgkm<10>(h0);
+    __builtin_amdgcn_sched_barrier(0);
+    MLTS_TMFMA4(h0, pfr[0][0])
+    softmax_half(I1{}, I0{}, s1, lse4);
+    MLTS_INTERLEAVE_4MFMA(5)
+    MLTS_TREAD8(h0, 2)
     wait_lgkm<8>(h1);
+    __builtin_amdgcn_sched_barrier(0);
     MLTS_TMFMA4(h1, pfr[0][1])
+    softmax_half(I1{}, I1{}, s1, lse4);
+    MLTS_INTERLEAVE_4MFMA(5)
     MLTS_TREAD8(h1, 3)
     lds_write_b128<2048>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][0]));
     lds_write_b128<3072>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][1]));
@@ -398,6 +419,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     MLTS_TMFMA4(h0, pfr[1][0])
     wait_lgkm<0>(h1);
     MLTS_TMFMA4(h1, pfr[1][1])
+#undef MLTS_INTERLEAVE_4MFMA
   };
 
   // ---- role 1, first half of a tile: dp = delta - dO V^T (kept in registers until P arrives) ----
