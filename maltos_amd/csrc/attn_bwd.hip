@@ -396,11 +396,11 @@ int mlts_attn_bwd_dq_bf16(const AttnBwdParams& bp, int D, int mode, hipStream_t 
 int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq);                          // attn_bwd_dma.hip
 int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);       // attn_bwd_dma.hip
 
-int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);     // attn_bwd_split.hip
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);  // attn_bwd_split.hip
 int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
 
 namespace {
-// dK/dV kernel for head_dim 128: the two-role kernel by default; tuning aid MLTS_BWD_VARIANT = "staged" (register
+// dK/dV kernel: the two-role kernel by default; tuning aid MLTS_BWD_VARIANT = "staged" (register
 // staged tiles, the head_dim 64 kernel) or "dma" (one role, one wavefront per SIMD) selects the earlier forms
 int dkdv_variant(int D) {
   static const int v = [] {
@@ -409,13 +409,14 @@ int dkdv_variant(int D) {
     if (e && e[0] == 'd') return 1;
     return 2;
   }();
-  return D == 128 ? v : 0;
+  if (D == 128) return v;
+  return v == 2 ? 2 : 0;  // head_dim 64 has the two-role and the register-staged forms
 }
 }  // namespace
 
 int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32) {
   (void)accumulate_f32;
-  return s->D == 128 ? mlts_attn_bwd_dkdv_dma_workspace(s->B, s->Hq, s->Sq) : 0;
+  return mlts_attn_bwd_dkdv_dma_workspace(s->B, s->Hq, s->Sq);  // lse2: B*Hq*Sq + 1 floats
 }
 
 int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
@@ -427,7 +428,7 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
   const int64_t lim = int64_t{1} << 24;
   if (p.qs[2] >= lim || p.ks[2] >= lim || p.vs[2] >= lim || bp.dos[2] >= lim) variant = 0;
   if (variant == 2) {
-    rc = mlts_attn_bwd_dkdv_bf16_split(bp, mode, workspace, st);
+    rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, workspace, st);
   } else if (variant == 1) {
     rc = mlts_attn_bwd_dkdv_bf16_dma(bp, mode, workspace, st);
   } else if (D == 128) {
@@ -440,6 +441,6 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
-  if (variant == 2) return mlts_attn_bwd_dq_bf16_tr(bp, mode, st);
+  if (variant == 2 && D == 128) return mlts_attn_bwd_dq_bf16_tr(bp, mode, st);
   return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

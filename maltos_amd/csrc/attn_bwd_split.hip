@@ -1,4 +1,4 @@
-// Attention backward, dK and dV, head_dim 128, bf16: two-role workgroup.
+// Attention backward, dK and dV, head_dim 64 and 128, bf16: two-role workgroup.
 //
 // A workgroup owns 128 keys of one (batch, kv head) and walks the 64-row query tiles that can see them (all
 // query heads of the GQA group), as attn_bwd.hip does, but its EIGHT wavefronts come in two roles per 32-key
@@ -22,26 +22,38 @@
 
 namespace {
 
-constexpr int D = 128;
 constexpr int BKV = 128;
 constexpr int BQ = 64;
 constexpr int WAVES = 8;
 constexpr int THREADS = WAVES * 64;
-constexpr int KS = D / 16;
-constexpr int DB = D / 32;
-constexpr int TILE_BYTES = BQ * D * 2;          // 16 KiB
-constexpr int STAT_OFF = 2 * TILE_BYTES;        // lse2[64] then delta[64], fp32
-constexpr int STAGE_BYTES = STAT_OFF + 2 * BQ * 4;
 constexpr int STAGES = 3;
-constexpr int PBUF_OFF = STAGES * STAGE_BYTES;  // P hand-over: [2 buffers][4 key blocks][4 fragments][64 lanes] x 16 B
-constexpr int PBUF_BYTES = 4 * 64 * 16;
-constexpr int LDS_BYTES = PBUF_OFF + 2 * 4 * PBUF_BYTES;
+constexpr int PBUF_BYTES = 4 * 64 * 16;  // P hand-over: [2 buffers][4 key blocks][4 fragments][64 lanes] x 16 B
 
+template <int D>
+struct SplitCfg {
+  static constexpr int KS = D / 16;                  // k-steps of the S / dP products
+  static constexpr int DB = D / 32;                  // 32-column blocks of dV / dK
+  static constexpr int RB = D * 2;                   // bytes per tile row
+  static constexpr int CPR = RB / 16;                // 16-byte chunks per row
+  static constexpr int TILE_BYTES = BQ * RB;
+  static constexpr int STAT_OFF = 2 * TILE_BYTES;    // lse2[64] then delta[64], fp32
+  static constexpr int STAGE_BYTES = STAT_OFF + 2 * BQ * 4;
+  static constexpr int PBUF_OFF = STAGES * STAGE_BYTES;
+  static constexpr int LDS_BYTES = PBUF_OFF + 2 * 4 * PBUF_BYTES;
+  static constexpr int NLD = BQ * CPR / THREADS;     // 16-byte chunks per thread and tile (2 or 1)
+};
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+// chunk swizzle of a tile row (depends on row & 15): chunk c of row r is stored at chunk c ^ swz(r).  256-byte rows:
+// swap of the two 2-bit halves; 128-byte rows (two rows per 256 bytes of banks): row bits 1,3,2 -> chunk bits 2,1,0.
+// Measured: ds_read_b128 of 32 consecutive rows ~215-250 B/clk/CU and the transpose reads ~155-160 B/clk/CU.
+template <int D>
+__device__ __forceinline__ int swz(int r) {
+  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (((r >> 1) & 1) << 2) | (((r >> 3) & 1) << 1) | ((r >> 2) & 1);
+}
 
 #define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define MLTS_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -99,8 +111,11 @@ __global__ __launch_bounds__(256) void lse2_kernel(const float* __restrict__ lse
   }
 }
 
-template <int MODE>
+template <int D, int MODE>
 __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const AttnBwdParams bp, const float* __restrict__ lse2) {
+  using C = SplitCfg<D>;
+  constexpr int KS = C::KS, DB = C::DB, RB = C::RB, CPR = C::CPR, TILE_BYTES = C::TILE_BYTES, STAT_OFF = C::STAT_OFF,
+                STAGE_BYTES = C::STAGE_BYTES, PBUF_OFF = C::PBUF_OFF, NLD = C::NLD;
   const AttnParams& p = bp.a;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -185,24 +200,24 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 
   // ---- tile loader.  Measured on gfx950: an LDS-DMA load keeps the LDS busy for about 27 cycles per KiB while its
   // data arrives (3-4 times a ds_write_b128 of the same data) and ds_read streams of the whole CU stall meanwhile, and
-  // this kernel is bound by LDS time.  So the next tile is fetched into registers right behind the barrier (64 bytes
-  // per thread: chunks t and t + 512 of the Q tile and of the dO tile, chunk c = row c/16, stored 16-byte slot c%16,
-  // source slot (c%16) ^ swz(row)) and written to LDS with ds_write_b128 after this tile's work.  Threads 0..127 also
+  // this kernel is bound by LDS time.  So the next tile is fetched into registers right behind the barrier (chunks
+  // t (and t + 512 for head_dim 128) of the Q tile and of the dO tile, chunk c = row c / CPR, stored 16-byte slot
+  // c % CPR, source slot (c % CPR) ^ swz(row)) and written to LDS with ds_write_b128 after this tile's work.  Threads 0..127 also
   // carry the 64 + 64 row statistics (lse2, delta). ----
   const int64_t lse2_inf = static_cast<int64_t>(p.B) * p.Hq * p.Sq;  // index of the +inf entry
   // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
   // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
-  int ld_row[2], ld_col[2];
-  uint32_t ld_qoff[2], ld_doff[2];
+  int ld_row[NLD], ld_col[NLD];
+  uint32_t ld_qoff[NLD], ld_doff[NLD];
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
+  for (int n = 0; n < NLD; ++n) {
     const int c = tid + n * THREADS;
-    ld_row[n] = c >> 4;
-    ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+    ld_row[n] = c / CPR;
+    ld_col[n] = ((c % CPR) ^ swz<D>((c / CPR) & 15)) * 8;
     ld_qoff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.qs[2]) + ld_col[n];
     ld_doff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(bp.dos[2]) + ld_col[n];
   }
-  v4i32 stg_q[2], stg_d[2];
+  v4i32 stg_q[NLD], stg_d[NLD];
   float stg_s = 0.f;
   const uint32_t lds0_ = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
   auto stage_load = [&](int it) {
@@ -212,7 +227,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1] + static_cast<int64_t>(q0) * bp.dos[2];
     const int last = p.Sq - 1 - q0;  // rows past the end repeat the last query; their lse2 is +inf
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < NLD; ++n) {
       uint32_t qo = ld_qoff[n], dofs = ld_doff[n];
       if (last < BQ - 1) {
         const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
@@ -232,9 +247,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   auto stage_store = [&](int stage) {
     const uint32_t a = stg_lane + stage * STAGE_BYTES;
     lds_write_b128<0>(a, stg_q[0]);
-    lds_write_b128<THREADS * 16>(a, stg_q[1]);
     lds_write_b128<TILE_BYTES>(a, stg_d[0]);
-    lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_d[1]);
+    if (NLD == 2) {
+      lds_write_b128<THREADS * 16>(a, stg_q[NLD - 1]);
+      lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_d[NLD - 1]);
+    }
     if (tid < 2 * BQ)
       asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(lds0_ + stage * STAGE_BYTES + tid * 4), "v"(stg_s), "n"(STAT_OFF));
   };
@@ -244,7 +261,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   int roff[KS];  // row-major fragment (A operand): row l32 (+32 qb), chunk 2 ks + hh; role 0 reads Q, role 1 dO
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
-    roff[ks] = role * TILE_BYTES + l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+    roff[ks] = role * TILE_BYTES + l32 * RB + (((ks * 2 + hh) ^ swz<D>(l32 & 15)) << 4);
   int toff[2][DB];  // transposed fragment halves: query row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16)
                     // + 4 (l16%4); role 0 reads dO^T, role 1 Q^T
 #pragma unroll
@@ -253,7 +270,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
-      toff[part][db] = (1 - role) * TILE_BYTES + rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+      toff[part][db] = (1 - role) * TILE_BYTES + rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
     }
   }
   // statistics of rows 32 qb + 8 g + 4 hh .. +3: role 0 reads lse2, role 1 delta
@@ -266,22 +283,28 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
 
-#define MLTS_RREAD4(dst, QB, KS0)                          \
-  dst[0] = lds_read_b128<(QB) * 8192>(ra[(KS0)]);          \
-  dst[1] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 1]);      \
-  dst[2] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 2]);      \
-  dst[3] = lds_read_b128<(QB) * 8192>(ra[(KS0) + 3]);
+#define MLTS_RREAD4(dst, QB, KS0)                              \
+  dst[0] = lds_read_b128<(QB) * 32 * RB>(ra[(KS0)]);           \
+  dst[1] = lds_read_b128<(QB) * 32 * RB>(ra[(KS0) + 1]);       \
+  dst[2] = lds_read_b128<(QB) * 32 * RB>(ra[(KS0) + 2]);       \
+  dst[3] = lds_read_b128<(QB) * 32 * RB>(ra[(KS0) + 3]);
 #define MLTS_RMFMA4(src, ACC, KS0)                                                                    \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) ACC =                                                 \
       __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[i]), kvf[(KS0) + i], ACC, 0, 0, 0);
-#define MLTS_TREAD8(dst, C)                                                  \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                        \
-    dst[2 * db] = lds_read_tr16_b64<(C) * 4096>(ta[0][db]);                  \
-    dst[2 * db + 1] = lds_read_tr16_b64<(C) * 4096>(ta[1][db]);              \
-  }
-#define MLTS_TMFMA4(src, AFRAG)                                                                                  \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) acc[db] =                                                    \
-      __builtin_amdgcn_mfma_f32_32x32x16_bf16(AFRAG, as_frag(src[2 * db], src[2 * db + 1]), acc[db], 0, 0, 0);
+  // a transposed group = eight reads / four MFMAs: one 16-query step c (head_dim 128, four column blocks) or the
+  // two steps c, c + 1 (head_dim 64, two column blocks each)
+#define MLTS_TREAD8(dst, CS)                                                          \
+  dst[0] = lds_read_tr16_b64<((CS) + 0 / DB) * 16 * RB>(ta[0][0 % DB]);               \
+  dst[1] = lds_read_tr16_b64<((CS) + 0 / DB) * 16 * RB>(ta[1][0 % DB]);               \
+  dst[2] = lds_read_tr16_b64<((CS) + 1 / DB) * 16 * RB>(ta[0][1 % DB]);               \
+  dst[3] = lds_read_tr16_b64<((CS) + 1 / DB) * 16 * RB>(ta[1][1 % DB]);               \
+  dst[4] = lds_read_tr16_b64<((CS) + 2 / DB) * 16 * RB>(ta[0][2 % DB]);               \
+  dst[5] = lds_read_tr16_b64<((CS) + 2 / DB) * 16 * RB>(ta[1][2 % DB]);               \
+  dst[6] = lds_read_tr16_b64<((CS) + 3 / DB) * 16 * RB>(ta[0][3 % DB]);               \
+  dst[7] = lds_read_tr16_b64<((CS) + 3 / DB) * 16 * RB>(ta[1][3 % DB]);
+#define MLTS_TMFMA4(src, AFRAG0, AFRAG1)                                                               \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) acc[u % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16( \
+      (u / DB) ? AFRAG1 : AFRAG0, as_frag(src[2 * u], src[2 * u + 1]), acc[u % DB], 0, 0, 0);
 
   // ---- role 0: one tile.  lane = key, accumulator register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4 ----
   auto role0_tile = [&](const bool masked, const int q0, const int stage, const int pbuf) {
@@ -368,57 +391,94 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     }
 #pragma unroll
     for (int g = 0; g < 4; ++g) st0[g] = lds_read_b128<0>(sa + g * 32);
-    MLTS_RREAD4(g0, 0, 0)
-    MLTS_RREAD4(g1, 0, 4)
-    wait_lgkm<8>(st0);
-    wait_lgkm<4>(g0);
-    MLTS_RMFMA4(g0, s0, 0)
+    // (whole-vector casts below: casting a single element of an asm result is miscompiled, element 0 is broadcast)
+    if constexpr (D == 128) {
+      MLTS_RREAD4(g0, 0, 0)
+      MLTS_RREAD4(g1, 0, 4)
+      wait_lgkm<8>(st0);
+      wait_lgkm<4>(g0);
+      MLTS_RMFMA4(g0, s0, 0)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) st1[g] = lds_read_b128<128>(sa + g * 32);
-    MLTS_RREAD4(g0, 1, 0)
-    wait_lgkm<8>(g1);
-    MLTS_RMFMA4(g1, s0, 4)
-    MLTS_RREAD4(g1, 1, 4)
-    wait_lgkm<8>(st1);
-    // whole-vector casts: casting a single element of an asm result is miscompiled (element 0 is broadcast)
+      for (int g = 0; g < 4; ++g) st1[g] = lds_read_b128<128>(sa + g * 32);
+      MLTS_RREAD4(g0, 1, 0)
+      wait_lgkm<8>(g1);
+      MLTS_RMFMA4(g1, s0, 4)
+      MLTS_RREAD4(g1, 1, 4)
+      wait_lgkm<8>(st1);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
-    if (masked) apply_mask(I0{}, s0);
-    wait_lgkm<4>(g0);
-    __builtin_amdgcn_sched_barrier(0);
-    MLTS_RMFMA4(g0, s1, 0)
-    softmax_half(I0{}, I0{}, s0, lse4);
-    MLTS_INTERLEAVE_4MFMA(5)
-    MLTS_TREAD8(h0, 0)
-    wait_lgkm<8>(g1);
-    __builtin_amdgcn_sched_barrier(0);
-    MLTS_RMFMA4(g1, s1, 4)
-    softmax_half(I0{}, I1{}, s0, lse4);
-    MLTS_INTERLEAVE_4MFMA(5)
-    MLTS_TREAD8(h1, 1)
-    lds_write_b128<0>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][0]));
-    lds_write_b128<1024>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][1]));
+      for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
+      if (masked) apply_mask(I0{}, s0);
+      wait_lgkm<4>(g0);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_RMFMA4(g0, s1, 0)
+      softmax_half(I0{}, I0{}, s0, lse4);
+      MLTS_INTERLEAVE_4MFMA(5)
+      MLTS_TREAD8(h0, 0)
+      wait_lgkm<8>(g1);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_RMFMA4(g1, s1, 4)
+      softmax_half(I0{}, I1{}, s0, lse4);
+      MLTS_INTERLEAVE_4MFMA(5)
+      MLTS_TREAD8(h1, 1)
+      lds_write_b128<0>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][0]));
+      lds_write_b128<1024>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][1]));
 #pragma unroll
-    for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
-    if (masked) apply_mask(I1{}, s1);
-    wait_lgkm<10>(h0);
-    __builtin_amdgcn_sched_barrier(0);
-    MLTS_TMFMA4(h0, pfr[0][0])
-    softmax_half(I1{}, I0{}, s1, lse4);
-    MLTS_INTERLEAVE_4MFMA(5)
-    MLTS_TREAD8(h0, 2)
-    wait_lgkm<8>(h1);
-    __builtin_amdgcn_sched_barrier(0);
-    MLTS_TMFMA4(h1, pfr[0][1])
-    softmax_half(I1{}, I1{}, s1, lse4);
-    MLTS_INTERLEAVE_4MFMA(5)
-    MLTS_TREAD8(h1, 3)
-    lds_write_b128<2048>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][0]));
-    lds_write_b128<3072>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][1]));
-    wait_lgkm<10>(h0);
-    MLTS_TMFMA4(h0, pfr[1][0])
-    wait_lgkm<0>(h1);
-    MLTS_TMFMA4(h1, pfr[1][1])
+      for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
+      if (masked) apply_mask(I1{}, s1);
+      wait_lgkm<10>(h0);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_TMFMA4(h0, pfr[0][0], pfr[0][0])
+      softmax_half(I1{}, I0{}, s1, lse4);
+      MLTS_INTERLEAVE_4MFMA(5)
+      MLTS_TREAD8(h0, 2)
+      wait_lgkm<8>(h1);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_TMFMA4(h1, pfr[0][1], pfr[0][1])
+      softmax_half(I1{}, I1{}, s1, lse4);
+      MLTS_INTERLEAVE_4MFMA(5)
+      MLTS_TREAD8(h1, 3)
+      lds_write_b128<2048>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][0]));
+      lds_write_b128<3072>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][1]));
+      wait_lgkm<10>(h0);
+      MLTS_TMFMA4(h0, pfr[1][0], pfr[1][0])
+      wait_lgkm<0>(h1);
+      MLTS_TMFMA4(h1, pfr[1][1], pfr[1][1])
+    } else {
+      // head_dim 64: one group of row reads per query block, one transposed group per two 16-query steps
+#pragma unroll
+      for (int g = 0; g < 4; ++g) st1[g] = lds_read_b128<128>(sa + g * 32);
+      MLTS_RREAD4(g0, 0, 0)
+      MLTS_RREAD4(g1, 1, 0)
+      wait_lgkm<8>(st0);  // twelve reads follow: st0 and st1 have both arrived
+      wait_lgkm<4>(g0);
+      MLTS_RMFMA4(g0, s0, 0)
+      MLTS_TREAD8(h0, 0)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st0[g]);
+      if (masked) apply_mask(I0{}, s0);
+      wait_lgkm<8>(g1);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_RMFMA4(g1, s1, 0)
+      softmax_half(I0{}, I0{}, s0, lse4);
+      softmax_half(I0{}, I1{}, s0, lse4);
+      MLTS_INTERLEAVE_4MFMA(10)
+      MLTS_TREAD8(h1, 2)
+      lds_write_b128<0>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][0]));
+      lds_write_b128<1024>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[0][1]));
+#pragma unroll
+      for (int g = 0; g < 4; ++g) lse4[g] = __builtin_bit_cast(f32x4, st1[g]);
+      if (masked) apply_mask(I1{}, s1);
+      wait_lgkm<10>(h0);
+      __builtin_amdgcn_sched_barrier(0);
+      MLTS_TMFMA4(h0, pfr[0][0], pfr[0][1])
+      softmax_half(I1{}, I0{}, s1, lse4);
+      softmax_half(I1{}, I1{}, s1, lse4);
+      MLTS_INTERLEAVE_4MFMA(10)
+      lds_write_b128<2048>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][0]));
+      lds_write_b128<3072>(pbuf_lane + pbuf, __builtin_bit_cast(v4i32, pfr[1][1]));
+      wait_lgkm<4>(h1);  // the four P writes follow it
+      MLTS_TMFMA4(h1, pfr[1][0], pfr[1][1])
+    }
 #undef MLTS_INTERLEAVE_4MFMA
   };
 
@@ -437,7 +497,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       st[4 + g] = lds_read_b128<128>(sa + g * 32);
     }
     MLTS_RREAD4(g0, 0, 0)
-    MLTS_RREAD4(g1, 0, 4)
+    if constexpr (D == 128) {
+      MLTS_RREAD4(g1, 0, 4)
+    } else {
+      MLTS_RREAD4(g1, 1, 0)
+    }
     wait_lgkm<8>(st);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -449,16 +513,23 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         dp1[g * 4 + r] = d1[r];
       }
     }
-    wait_lgkm<4>(g0);
-    MLTS_RMFMA4(g0, dp0, 0)
-    MLTS_RREAD4(g0, 1, 0)
-    wait_lgkm<4>(g1);
-    MLTS_RMFMA4(g1, dp0, 4)
-    MLTS_RREAD4(g1, 1, 4)
-    wait_lgkm<4>(g0);
-    MLTS_RMFMA4(g0, dp1, 0)
-    wait_lgkm<0>(g1);
-    MLTS_RMFMA4(g1, dp1, 4)
+    if constexpr (D == 128) {
+      wait_lgkm<4>(g0);
+      MLTS_RMFMA4(g0, dp0, 0)
+      MLTS_RREAD4(g0, 1, 0)
+      wait_lgkm<4>(g1);
+      MLTS_RMFMA4(g1, dp0, 4)
+      MLTS_RREAD4(g1, 1, 4)
+      wait_lgkm<4>(g0);
+      MLTS_RMFMA4(g0, dp1, 0)
+      wait_lgkm<0>(g1);
+      MLTS_RMFMA4(g1, dp1, 4)
+    } else {
+      wait_lgkm<4>(g0);
+      MLTS_RMFMA4(g0, dp0, 0)
+      wait_lgkm<0>(g1);
+      MLTS_RMFMA4(g1, dp1, 0)
+    }
   };
   // ---- role 1, one barrier later: -dS = P dp as soon as P has arrived (frees dp for the next tile) ... ----
   bf16x8 dsfr[4];
@@ -492,18 +563,27 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 #pragma unroll
       for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
     v2i32 h0[8], h1[8];
-    MLTS_TREAD8(h0, 0)
-    MLTS_TREAD8(h1, 1)
-    wait_lgkm<8>(h0);
-    MLTS_TMFMA4(h0, dsfr[0])
-    MLTS_TREAD8(h0, 2)
-    wait_lgkm<8>(h1);
-    MLTS_TMFMA4(h1, dsfr[1])
-    MLTS_TREAD8(h1, 3)
-    wait_lgkm<8>(h0);
-    MLTS_TMFMA4(h0, dsfr[2])
-    wait_lgkm<0>(h1);
-    MLTS_TMFMA4(h1, dsfr[3])
+    if constexpr (D == 128) {
+      MLTS_TREAD8(h0, 0)
+      MLTS_TREAD8(h1, 1)
+      wait_lgkm<8>(h0);
+      MLTS_TMFMA4(h0, dsfr[0], dsfr[0])
+      MLTS_TREAD8(h0, 2)
+      wait_lgkm<8>(h1);
+      MLTS_TMFMA4(h1, dsfr[1], dsfr[1])
+      MLTS_TREAD8(h1, 3)
+      wait_lgkm<8>(h0);
+      MLTS_TMFMA4(h0, dsfr[2], dsfr[2])
+      wait_lgkm<0>(h1);
+      MLTS_TMFMA4(h1, dsfr[3], dsfr[3])
+    } else {
+      MLTS_TREAD8(h0, 0)
+      MLTS_TREAD8(h1, 2)
+      wait_lgkm<8>(h0);
+      MLTS_TMFMA4(h0, dsfr[0], dsfr[1])
+      wait_lgkm<0>(h1);
+      MLTS_TMFMA4(h1, dsfr[2], dsfr[3])
+    }
   };
 #undef MLTS_RREAD4
 #undef MLTS_RMFMA4
@@ -577,14 +657,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   }
 }
 
-template <int MODE>
+template <int D, int MODE>
 int launch(const AttnBwdParams& bp, const float* lse2, hipStream_t st) {
-  auto kern = attn_bwd_dkdv_split_kernel<MODE>;
+  auto kern = attn_bwd_dkdv_split_kernel<D, MODE>;
+  constexpr int lds_bytes = SplitCfg<D>::LDS_BYTES;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
       return MLTS_ERR_LAUNCH;
     }
     configured = true;
@@ -592,21 +673,26 @@ int launch(const AttnBwdParams& bp, const float* lse2, hipStream_t st) {
   const int64_t blocks = static_cast<int64_t>(bp.nkt) * bp.a.B * bp.a.Hkv;
   if (blocks > 0) {
     MltsKernelTimer timer("attn_bwd_dkdv", st);
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, bp, lse2);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), lds_bytes, st, bp, lse2);
   }
   return mlts_check_launch("mlts_attn_bwd");
 }
 
+template <int D>
+int launch_mode(const AttnBwdParams& bp, int mode, const float* lse2, hipStream_t st) {
+  if (mode == MLTS_MASK_NONE) return launch<D, MLTS_MASK_NONE>(bp, lse2, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<D, MLTS_MASK_CAUSAL>(bp, lse2, st);
+  return launch<D, MLTS_MASK_DOC>(bp, lse2, st);
+}
+
 }  // namespace
 
-// head_dim 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
-int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int mode, void* workspace, hipStream_t st) {
+// head_dim 64 or 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   float* lse2 = static_cast<float*>(workspace);
   const int64_t n = static_cast<int64_t>(p.B) * p.Hq * p.Sq;
   hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 256) / 256)), dim3(256), 0, st, p.lse, lse2, n);
-  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(bp, lse2, st);
-  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(bp, lse2, st);
-  return launch<MLTS_MASK_DOC>(bp, lse2, st);
+  return D == 128 ? launch_mode<128>(bp, mode, lse2, st) : launch_mode<64>(bp, mode, lse2, st);
 }
