@@ -397,7 +397,7 @@ int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq);    
 int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);       // attn_bwd_dma.hip
 
 int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);  // attn_bwd_split.hip
-int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
+int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
 
 namespace {
 // dK/dV kernel: the two-role kernel by default; tuning aid MLTS_BWD_VARIANT = "staged" (register
@@ -441,6 +441,6 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
-  if (variant == 2 && D == 128) return mlts_attn_bwd_dq_bf16_tr(bp, mode, st);
+  if (variant == 2) return mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
   return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

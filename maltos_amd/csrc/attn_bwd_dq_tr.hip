@@ -1,4 +1,4 @@
-// Attention backward, dQ, head_dim 128, bf16: the version of attn_bwd_dq.hip with one LDS copy per tile.
+// Attention backward, dQ, head_dim 64 and 128, bf16: the version of attn_bwd_dq.hip with one LDS copy per tile.
 //
 // Same decomposition (a workgroup of 8 wavefronts owns 256 query rows of one (batch, head), each wavefront 32 of
 // them, Q and dO stay in registers, it walks the visible keys in tiles of 64 and recomputes the scores transposed so
@@ -15,22 +15,34 @@
 
 namespace {
 
-constexpr int D = 128;
 constexpr int BN = 64;
 constexpr int WAVES = 8;
 constexpr int THREADS = WAVES * 64;
 constexpr int BM = WAVES * 32;
-constexpr int KS = D / 16;
-constexpr int DB = D / 32;
-constexpr int TILE_BYTES = BN * D * 2;       // 16 KiB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K then V
 constexpr int STAGES = 2;
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+
+template <int D>
+struct DqCfg {
+  static constexpr int KS = D / 16;
+  static constexpr int DB = D / 32;
+  static constexpr int RB = D * 2;                     // bytes per tile row
+  static constexpr int CPR = RB / 16;                  // 16-byte chunks per row
+  static constexpr int TILE_BYTES = BN * RB;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int NLD = BN * CPR / THREADS;       // 16-byte chunks per thread and tile (2 or 1)
+};
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef int v2i32 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+// chunk swizzle of a tile row (see attn_bwd_split.hip): 256-byte rows swap the 2-bit halves of row & 15, 128-byte rows
+// send row bits 1,3,2 to chunk bits 2,1,0
+template <int D>
+__device__ __forceinline__ int swz(int r) {
+  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (((r >> 1) & 1) << 2) | (((r >> 3) & 1) << 1) | ((r >> 2) & 1);
+}
 
 #define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -76,8 +88,11 @@ __device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
   return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
 }
 
-template <int MODE>
+template <int D, int MODE>
 __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdParams bp) {
+  using C = DqCfg<D>;
+  constexpr int KS = C::KS, DB = C::DB, RB = C::RB, CPR = C::CPR, TILE_BYTES = C::TILE_BYTES, STAGE_BYTES = C::STAGE_BYTES,
+                NLD = C::NLD;
   const AttnParams& p = bp.a;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -158,24 +173,24 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   // stored 16-byte slot c%16, source slot (c%16) ^ swz(row)); registers now, ds_write_b128 after this tile's work ----
   // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
   // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
-  int ld_row[2], ld_col[2];
-  uint32_t ld_koff[2], ld_voff[2];
+  int ld_row[NLD], ld_col[NLD];
+  uint32_t ld_koff[NLD], ld_voff[NLD];
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
+  for (int n = 0; n < NLD; ++n) {
     const int c = tid + n * THREADS;
-    ld_row[n] = c >> 4;
-    ld_col[n] = ((c & 15) ^ swz4((c >> 4) & 15)) * 8;
+    ld_row[n] = c / CPR;
+    ld_col[n] = ((c % CPR) ^ swz<D>((c / CPR) & 15)) * 8;
     ld_koff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.ks[2]) + ld_col[n];
     ld_voff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n];
   }
-  v4i32 stg_k[2], stg_v[2];
+  v4i32 stg_k[NLD], stg_v[NLD];
   auto stage_load = [&](int j) {
     const int kv0 = j * BN;
     const bf16_t* Kt = K + static_cast<int64_t>(kv0) * p.ks[2];
     const bf16_t* Vt = V + static_cast<int64_t>(kv0) * p.vs[2];
     const int last = p.Sk - 1 - kv0;  // rows past the end repeat the last key; their scores are masked
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < NLD; ++n) {
       uint32_t ko = ld_koff[n], vo = ld_voff[n];
       if (last < BN - 1) {
         const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
@@ -190,16 +205,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   auto stage_store = [&](int stage) {
     const uint32_t a = lds0 + stage * STAGE_BYTES + tid * 16;
     lds_write_b128<0>(a, stg_k[0]);
-    lds_write_b128<THREADS * 16>(a, stg_k[1]);
     lds_write_b128<TILE_BYTES>(a, stg_v[0]);
-    lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_v[1]);
+    if (NLD == 2) {
+      lds_write_b128<THREADS * 16>(a, stg_k[NLD - 1]);
+      lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_v[NLD - 1]);
+    }
   };
 
   // ---- per-lane LDS read offsets (tile invariant) ----
   // (LDS addresses of stage 0; the stage, the key block and the tile are added as instruction offsets)
   uint32_t ra[KS];  // row-major fragment (A operand): row l32 (+32 kb), chunk 2 ks + hh
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + l32 * RB + (((ks * 2 + hh) ^ swz<D>(l32 & 15)) << 4);
   uint32_t ta[2][DB];  // K^T fragment halves: key row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4)
 #pragma unroll
   for (int part = 0; part < 2; ++part) {
@@ -207,7 +224,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
-      ta[part][db] = lds0 + rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+      ta[part][db] = lds0 + rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
     }
   }
 
@@ -220,16 +237,16 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   // read groups are kept small (two 16-byte row reads, or four transpose reads) and two are in flight: the kernel
   // sits at the 256-register limit of two wavefronts per SIMD
 #define MLTS_RREAD2(dst, KB, KS0)                                                  \
-  dst[0] = lds_read_b128<(KB) * 8192>(ra[(KS0)] + so);                             \
-  dst[1] = lds_read_b128<TILE_BYTES + (KB) * 8192>(ra[(KS0)] + so);
+  dst[0] = lds_read_b128<(KB) * 32 * RB>(ra[(KS0)] + so);                             \
+  dst[1] = lds_read_b128<TILE_BYTES + (KB) * 32 * RB>(ra[(KS0)] + so);
 #define MLTS_SMFMA2(src, KS0)                                                                            \
   s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), qf[(KS0)], s, 0, 0, 0);                   \
   dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), ndof[(KS0)], dp, 0, 0, 0);
 #define MLTS_TREAD4(dst, C, H)                                                       \
-  dst[0] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H)] + so);                       \
-  dst[1] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H)] + so);                       \
-  dst[2] = lds_read_tr16_b64<(C) * 4096>(ta[0][2 * (H) + 1] + so);                   \
-  dst[3] = lds_read_tr16_b64<(C) * 4096>(ta[1][2 * (H) + 1] + so);
+  dst[0] = lds_read_tr16_b64<(C) * 16 * RB>(ta[0][2 * (H)] + so);                       \
+  dst[1] = lds_read_tr16_b64<(C) * 16 * RB>(ta[1][2 * (H)] + so);                       \
+  dst[2] = lds_read_tr16_b64<(C) * 16 * RB>(ta[0][2 * (H) + 1] + so);                   \
+  dst[3] = lds_read_tr16_b64<(C) * 16 * RB>(ta[1][2 * (H) + 1] + so);
 #define MLTS_TMFMA2(src, H, BFRAG)                                                                                        \
   dqacc[2 * (H)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0], src[1]), BFRAG, dqacc[2 * (H)], 0, 0, 0);       \
   dqacc[2 * (H) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2], src[3]), BFRAG, dqacc[2 * (H) + 1], 0, 0, 0);
@@ -289,7 +306,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     };
     v4i32 g0[2], g1[2];
     v2i32 h0[4], h1[4];
-#define MLTS_KEY_BLOCK(KB)                                                         \
+#define MLTS_KEY_BLOCK_128(KB)                                                     \
     acc_init();                                                                    \
     MLTS_RREAD2(g0, KB, 0)                                                         \
     MLTS_RREAD2(g1, KB, 1)                                                         \
@@ -306,9 +323,26 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     wait_lgkm<4>(h1); MLTS_TMFMA2(h1, 1, dsf[0]) MLTS_TREAD4(h1, 2 * (KB) + 1, 1)  \
     wait_lgkm<4>(h0); MLTS_TMFMA2(h0, 0, dsf[1])                                   \
     wait_lgkm<0>(h1); MLTS_TMFMA2(h1, 1, dsf[1])
-    MLTS_KEY_BLOCK(0)
-    MLTS_KEY_BLOCK(1)
-#undef MLTS_KEY_BLOCK
+#define MLTS_KEY_BLOCK_64(KB)                                                      \
+    acc_init();                                                                    \
+    MLTS_RREAD2(g0, KB, 0)                                                         \
+    MLTS_RREAD2(g1, KB, 1)                                                         \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 0) MLTS_RREAD2(g0, KB, 2)                    \
+    wait_lgkm<2>(g1); MLTS_SMFMA2(g1, 1) MLTS_RREAD2(g1, KB, 3)                    \
+    wait_lgkm<2>(g0); MLTS_SMFMA2(g0, 2) MLTS_TREAD4(h0, 2 * (KB), 0)              \
+    wait_lgkm<4>(g1); MLTS_SMFMA2(g1, 3) MLTS_TREAD4(h1, 2 * (KB) + 1, 0)          \
+    ds_block(KB);                                                                  \
+    wait_lgkm<4>(h0); MLTS_TMFMA2(h0, 0, dsf[0])                                   \
+    wait_lgkm<0>(h1); MLTS_TMFMA2(h1, 0, dsf[1])
+    if constexpr (D == 128) {
+      MLTS_KEY_BLOCK_128(0)
+      MLTS_KEY_BLOCK_128(1)
+    } else {
+      MLTS_KEY_BLOCK_64(0)
+      MLTS_KEY_BLOCK_64(1)
+    }
+#undef MLTS_KEY_BLOCK_128
+#undef MLTS_KEY_BLOCK_64
   };
 #undef MLTS_RREAD2
 #undef MLTS_SMFMA2
@@ -373,14 +407,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   }
 }
 
-template <int MODE>
+template <int D, int MODE>
 int launch(AttnBwdParams bp, hipStream_t st) {
-  auto kern = attn_bwd_dq_tr_kernel<MODE>;
+  auto kern = attn_bwd_dq_tr_kernel<D, MODE>;
+  constexpr int lds_bytes = DqCfg<D>::LDS_BYTES;
   static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+  if (!configured && lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
       return MLTS_ERR_LAUNCH;
     }
     configured = true;
@@ -389,16 +424,21 @@ int launch(AttnBwdParams bp, hipStream_t st) {
   const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * bp.a.Hq;
   if (blocks > 0) {
     MltsKernelTimer timer("attn_bwd_dq", st);
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, bp);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), lds_bytes, st, bp);
   }
   return mlts_check_launch("mlts_attn_bwd");
 }
 
+template <int D>
+int launch_mode(const AttnBwdParams& bp, int mode, hipStream_t st) {
+  if (mode == MLTS_MASK_NONE) return launch<D, MLTS_MASK_NONE>(bp, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<D, MLTS_MASK_CAUSAL>(bp, st);
+  return launch<D, MLTS_MASK_DOC>(bp, st);
+}
+
 }  // namespace
 
-// head_dim 128, Sk >= 1 when Sq >= 1 reaches a key, 16-byte aligned rows (checked by the caller)
-int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int mode, hipStream_t st) {
-  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(bp, st);
-  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(bp, st);
-  return launch<MLTS_MASK_DOC>(bp, st);
+// head_dim 64 or 128, 16-byte aligned rows (checked by the caller)
+int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st) {
+  return D == 128 ? launch_mode<128>(bp, mode, st) : launch_mode<64>(bp, mode, st);
 }
