@@ -452,11 +452,11 @@ int dispatch_fwd(AttnParams p, int D, int mode, hipStream_t st) {
 }
 }  // namespace
 
-int mlts_attn_fwd_bf16_dma(const AttnParams& p, int mode, hipStream_t st);  // attn_fwd_dma.hip
+int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st);  // attn_fwd_dma.hip
 
 int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st) {
   // tuning aid: MLTS_FWD_VARIANT = "4x2" (one wavefront per SIMD) or "8x1" (register-staged tiles) selects the
-  // older forms for head_dim 128; the default for head_dim 128 is the LDS-DMA pipeline
+  // older forms; the default is the LDS-DMA pipeline
   static const int variant = [] {
     const char* e = getenv("MLTS_FWD_VARIANT");
     if (e && e[0] == '4') return 4;
@@ -464,6 +464,6 @@ int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st) {
     return 0;
   }();
   if (variant == 4) return dispatch_fwd<4, 2>(p, D, mode, st);
-  if (variant == 0 && D == 128) return mlts_attn_fwd_bf16_dma(p, mode, st);
+  if (variant == 0) return mlts_attn_fwd_bf16_dma(p, D, mode, st);
   return dispatch_fwd<8, 1>(p, D, mode, st);
 }

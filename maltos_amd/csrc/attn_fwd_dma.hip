@@ -1,4 +1,4 @@
-// Attention forward, head_dim 128, bf16: the gfx950 memory pipeline version.
+// Attention forward, head_dim 64 and 128, bf16: the gfx950 memory pipeline version.
 //
 // Same math and register layouts as attn_fwd.hip (S^T = K Q^T, P in registers, O^T = V^T P^T, eight
 // wavefronts x 32 query rows), but K and V tiles travel global -> LDS with the 16-byte LDS-DMA loads
@@ -15,21 +15,32 @@
 
 namespace {
 
-constexpr int D = 128;
 constexpr int BN = 64;
 constexpr int WAVES = 8;
 constexpr int THREADS = WAVES * 64;
 constexpr int BM = WAVES * 32;
-constexpr int KS = D / 16;
-constexpr int DB = D / 32;
-constexpr int TILE_BYTES = BN * D * 2;       // 16 KiB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K then V
 constexpr int STAGES = 4;
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-constexpr int LOADS_PER_TILE = 2 * TILE_BYTES / (WAVES * 1024);  // DMA instructions per wavefront per stage (4)
 
+template <int D>
+struct FwdCfg {
+  static constexpr int KS = D / 16;
+  static constexpr int DB = D / 32;
+  static constexpr int RB = D * 2;                     // bytes per tile row
+  static constexpr int CPR = RB / 16;                  // 16-byte chunks per row
+  static constexpr int TILE_BYTES = BN * RB;
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int PPW = TILE_BYTES / (WAVES * 1024);  // 1 KiB pieces of each tile per wavefront (2 or 1)
+  static constexpr int LOADS_PER_TILE = 2 * PPW;           // DMA instructions per wavefront per stage
+};
 
-__device__ __forceinline__ int swz4(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+// chunk swizzle of a tile row (depends on row & 15): 256-byte rows swap the two 2-bit halves; 128-byte rows (two rows
+// per 256 bytes of banks) send row bits 1,3,2 to chunk bits 2,1,0
+template <int D>
+__device__ __forceinline__ int swz(int r) {
+  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (((r >> 1) & 1) << 2) | (((r >> 3) & 1) << 1) | ((r >> 2) & 1);
+}
 
 #define MLTS_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define MLTS_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -75,8 +86,11 @@ __device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
   return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
 }
 
-template <int MODE>
+template <int D, int MODE>
 __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams p) {
+  using C = FwdCfg<D>;
+  constexpr int KS = C::KS, DB = C::DB, RB = C::RB, CPR = C::CPR, TILE_BYTES = C::TILE_BYTES, STAGE_BYTES = C::STAGE_BYTES,
+                PPW = C::PPW, LOADS_PER_TILE = C::LOADS_PER_TILE;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
@@ -146,25 +160,25 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     return j;
   };
 
-  // ---- DMA loader: this wavefront moves 1 KiB pieces 2w, 2w+1 of the K tile and of the V tile ----
-  // piece n holds rows 4n .. 4n+3; lane L -> row 4n + L/16, stored chunk L%16, source chunk (L%16) ^ swz(row)
-  int ld_row[2], ld_col[2];
+  // ---- DMA loader: this wavefront moves PPW 1 KiB pieces of the K tile and of the V tile; piece n holds rows
+  // n * 64 / CPR ..; lane L -> row n * 64 / CPR + L / CPR, stored chunk L % CPR, source chunk (L % CPR) ^ swz(row) ----
+  int ld_row[PPW], ld_col[PPW];
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
-    const int row = (wave * 2 + n) * 4 + (lane >> 4);
+  for (int n = 0; n < PPW; ++n) {
+    const int row = (wave * PPW + n) * (64 / CPR) + lane / CPR;
     ld_row[n] = row;
-    ld_col[n] = ((lane & 15) ^ swz4(row & 15)) * 8;
+    ld_col[n] = ((lane % CPR) ^ swz<D>(row & 15)) * 8;
   }
   auto issue_tile = [&](int j, int stage) {
     const int kv0 = j * BN;
     unsigned char* sbase = smem + stage * STAGE_BYTES;
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < PPW; ++n) {
       const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
       const bf16_t* ksrc = K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n];
       const bf16_t* vsrc = V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n];
-      __builtin_amdgcn_global_load_lds(MLTS_GLB(ksrc), MLTS_LDS(sbase + (wave * 2 + n) * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(MLTS_GLB(vsrc), MLTS_LDS(sbase + TILE_BYTES + (wave * 2 + n) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(MLTS_GLB(ksrc), MLTS_LDS(sbase + (wave * PPW + n) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(MLTS_GLB(vsrc), MLTS_LDS(sbase + TILE_BYTES + (wave * PPW + n) * 1024), 16, 0, 0);
     }
   };
 
@@ -172,7 +186,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
   int koff[KS];   // K fragment (A operand of S^T): row l32 (+32 kb), chunk 2 ks + hh
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) koff[ks] = l32 * 256 + (((ks * 2 + hh) ^ swz4(l32 & 15)) << 4);
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = l32 * RB + (((ks * 2 + hh) ^ swz<D>(l32 & 15)) << 4);
   int voff[2][DB];  // V^T fragment halves: key row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4)
 #pragma unroll
   for (int part = 0; part < 2; ++part) {
@@ -180,7 +194,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
-      voff[part][db] = rlow * 256 + (((col >> 3) ^ swz4(rlow)) << 4) + ((col >> 2) & 1) * 8;
+      voff[part][db] = rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
     }
   }
 
@@ -234,26 +248,41 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 #pragma unroll
           for (int db = 0; db < DB; ++db) va[part][db] = sb + voff[part][db];
         v2i32 h0[8], h1[8];
-#define MLTS_VREAD8(dst, C)                                                                 \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) {                                       \
-    dst[2 * db] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[0][db]);                    \
-    dst[2 * db + 1] = lds_read_tr16_b64<TILE_BYTES + (C) * 4096>(va[1][db]);                \
-  }
-#define MLTS_VMFMA4(src, C)                                                                                     \
-  _Pragma("unroll") for (int db = 0; db < DB; ++db) oacc[db] =                                                  \
-      __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2 * db], src[2 * db + 1]), pf[C], oacc[db], 0, 0, 0);
-        MLTS_VREAD8(h0, 0)
-        MLTS_VREAD8(h1, 1)
-        wait_lgkm<8>(h0);
-        MLTS_VMFMA4(h0, 0)
-        MLTS_VREAD8(h0, 2)
-        wait_lgkm<8>(h1);
-        MLTS_VMFMA4(h1, 1)
-        MLTS_VREAD8(h1, 3)
-        wait_lgkm<8>(h0);
-        MLTS_VMFMA4(h0, 2)
-        wait_lgkm<0>(h1);
-        MLTS_VMFMA4(h1, 3)
+        // a group = eight transpose reads / four MFMAs: one 16-key step c (head_dim 128, four column blocks) or the
+        // two steps c, c + 1 (head_dim 64, two column blocks each)
+#define MLTS_VREAD8(dst, CS)                                                                   \
+  dst[0] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 0 / DB) * 16 * RB>(va[0][0 % DB]);           \
+  dst[1] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 0 / DB) * 16 * RB>(va[1][0 % DB]);           \
+  dst[2] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 1 / DB) * 16 * RB>(va[0][1 % DB]);           \
+  dst[3] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 1 / DB) * 16 * RB>(va[1][1 % DB]);           \
+  dst[4] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 2 / DB) * 16 * RB>(va[0][2 % DB]);           \
+  dst[5] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 2 / DB) * 16 * RB>(va[1][2 % DB]);           \
+  dst[6] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 3 / DB) * 16 * RB>(va[0][3 % DB]);           \
+  dst[7] = lds_read_tr16_b64<TILE_BYTES + ((CS) + 3 / DB) * 16 * RB>(va[1][3 % DB]);
+#define MLTS_VMFMA4(src, CS)                                                                                 \
+  _Pragma("unroll") for (int u = 0; u < 4; ++u) oacc[u % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(      \
+      as_frag(src[2 * u], src[2 * u + 1]), pf[(CS) + u / DB], oacc[u % DB], 0, 0, 0);
+        if constexpr (D == 128) {
+          MLTS_VREAD8(h0, 0)
+          MLTS_VREAD8(h1, 1)
+          wait_lgkm<8>(h0);
+          MLTS_VMFMA4(h0, 0)
+          MLTS_VREAD8(h0, 2)
+          wait_lgkm<8>(h1);
+          MLTS_VMFMA4(h1, 1)
+          MLTS_VREAD8(h1, 3)
+          wait_lgkm<8>(h0);
+          MLTS_VMFMA4(h0, 2)
+          wait_lgkm<0>(h1);
+          MLTS_VMFMA4(h1, 3)
+        } else {
+          MLTS_VREAD8(h0, 0)
+          MLTS_VREAD8(h1, 2)
+          wait_lgkm<8>(h0);
+          MLTS_VMFMA4(h0, 0)
+          wait_lgkm<0>(h1);
+          MLTS_VMFMA4(h1, 2)
+        }
 #undef MLTS_VREAD8
 #undef MLTS_VMFMA4
       }
@@ -291,25 +320,34 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
         // sixteen K fragments in four groups of four, two groups in flight
         v4i32 g0[4], g1[4];
 #define MLTS_KREAD4(dst, KB, KS0)                                   \
-  dst[0] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 0]);               \
-  dst[1] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 1]);               \
-  dst[2] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 2]);               \
-  dst[3] = lds_read_b128<(KB) * 8192>(ka[(KS0) + 3]);
+  dst[0] = lds_read_b128<(KB) * 32 * RB>(ka[(KS0) + 0]);               \
+  dst[1] = lds_read_b128<(KB) * 32 * RB>(ka[(KS0) + 1]);               \
+  dst[2] = lds_read_b128<(KB) * 32 * RB>(ka[(KS0) + 2]);               \
+  dst[3] = lds_read_b128<(KB) * 32 * RB>(ka[(KS0) + 3]);
 #define MLTS_KMFMA4(src, KB, KS0)                                                                              \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) sacc[KB] =                                                     \
       __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[i]), qf[(KS0) + i], sacc[KB], 0, 0, 0);
-        MLTS_KREAD4(g0, 0, 0)
-        MLTS_KREAD4(g1, 0, 4)
-        wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
-        MLTS_KMFMA4(g0, 0, 0)
-        MLTS_KREAD4(g0, 1, 0)
-        wait_lgkm<4>(g1[0], g1[1], g1[2], g1[3]);
-        MLTS_KMFMA4(g1, 0, 4)
-        MLTS_KREAD4(g1, 1, 4)
-        wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
-        MLTS_KMFMA4(g0, 1, 0)
-        wait_lgkm<0>(g1[0], g1[1], g1[2], g1[3]);
-        MLTS_KMFMA4(g1, 1, 4)
+        if constexpr (D == 128) {
+          MLTS_KREAD4(g0, 0, 0)
+          MLTS_KREAD4(g1, 0, 4)
+          wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
+          MLTS_KMFMA4(g0, 0, 0)
+          MLTS_KREAD4(g0, 1, 0)
+          wait_lgkm<4>(g1[0], g1[1], g1[2], g1[3]);
+          MLTS_KMFMA4(g1, 0, 4)
+          MLTS_KREAD4(g1, 1, 4)
+          wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
+          MLTS_KMFMA4(g0, 1, 0)
+          wait_lgkm<0>(g1[0], g1[1], g1[2], g1[3]);
+          MLTS_KMFMA4(g1, 1, 4)
+        } else {
+          MLTS_KREAD4(g0, 0, 0)
+          MLTS_KREAD4(g1, 1, 0)
+          wait_lgkm<4>(g0[0], g0[1], g0[2], g0[3]);
+          MLTS_KMFMA4(g0, 0, 0)
+          wait_lgkm<0>(g1[0], g1[1], g1[2], g1[3]);
+          MLTS_KMFMA4(g1, 1, 0)
+        }
 #undef MLTS_KREAD4
 #undef MLTS_KMFMA4
       }
@@ -408,14 +446,15 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   }
 }
 
-template <int MODE>
+template <int D, int MODE>
 int launch(AttnParams p, hipStream_t st) {
-  auto kern = attn_fwd_dma_kernel<MODE>;
+  auto kern = attn_fwd_dma_kernel<D, MODE>;
+  constexpr int lds_bytes = FwdCfg<D>::LDS_BYTES;
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+      mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
       return MLTS_ERR_LAUNCH;
     }
     configured = true;
@@ -424,16 +463,21 @@ int launch(AttnParams p, hipStream_t st) {
   const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * p.Hq;
   {
     MltsKernelTimer timer("attn_fwd", st);
-    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), LDS_BYTES, st, p);
+    hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), lds_bytes, st, p);
   }
   return mlts_check_launch("mlts_attn_fwd");
 }
 
+template <int D>
+int launch_mode(const AttnParams& p, int mode, hipStream_t st) {
+  if (mode == MLTS_MASK_NONE) return launch<D, MLTS_MASK_NONE>(p, st);
+  if (mode == MLTS_MASK_CAUSAL) return launch<D, MLTS_MASK_CAUSAL>(p, st);
+  return launch<D, MLTS_MASK_DOC>(p, st);
+}
+
 }  // namespace
 
-// Requires head_dim 128, Sk >= 1 and 16-byte aligned rows (checked by the caller).
-int mlts_attn_fwd_bf16_dma(const AttnParams& p, int mode, hipStream_t st) {
-  if (mode == MLTS_MASK_NONE) return launch<MLTS_MASK_NONE>(p, st);
-  if (mode == MLTS_MASK_CAUSAL) return launch<MLTS_MASK_CAUSAL>(p, st);
-  return launch<MLTS_MASK_DOC>(p, st);
+// Requires head_dim 64 or 128, Sk >= 1 and 16-byte aligned rows (checked by the caller).
+int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st) {
+  return D == 128 ? launch_mode<128>(p, mode, st) : launch_mode<64>(p, mode, st);
 }
