@@ -240,7 +240,7 @@ def main() -> int:
     if not args.skip_extra:
         extra = {}
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
-        extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(2, args.warmup // 2))
+        extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(5, args.warmup))
         result["extra"] = extra
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)

@@ -393,44 +393,37 @@ int launch_bwd(const AttnBwdParams& bp, hipStream_t st) {
 
 int mlts_attn_bwd_dq_bf16(const AttnBwdParams& bp, int D, int mode, hipStream_t st);
 
-int64_t mlts_attn_bwd_dkdv_dma_workspace(int64_t B, int64_t Hq, int64_t Sq);                          // attn_bwd_dma.hip
-int mlts_attn_bwd_dkdv_bf16_dma(AttnBwdParams bp, int mode, void* workspace, hipStream_t st);       // attn_bwd_dma.hip
+int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq);                           // attn_bwd_split.hip
 
 int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);  // attn_bwd_split.hip
 int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
 
 namespace {
-// dK/dV kernel: the two-role kernel by default; tuning aid MLTS_BWD_VARIANT = "staged" (register
-// staged tiles, the head_dim 64 kernel) or "dma" (one role, one wavefront per SIMD) selects the earlier forms
-int dkdv_variant(int D) {
-  static const int v = [] {
+// Two-role dK/dV kernel and transpose-read dQ kernel by default; tuning aid MLTS_BWD_VARIANT=staged selects the
+// register-staged kernels of this file and attn_bwd_dq.hip (also the fallback for very large row strides).
+bool use_staged_bwd() {
+  static const bool staged = [] {
     const char* e = getenv("MLTS_BWD_VARIANT");
-    if (e && e[0] == 's') return 0;
-    if (e && e[0] == 'd') return 1;
-    return 2;
+    return e && e[0] == 's';
   }();
-  if (D == 128) return v;
-  return v == 2 ? 2 : 0;  // head_dim 64 has the two-role and the register-staged forms
+  return staged;
 }
 }  // namespace
 
 int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32) {
   (void)accumulate_f32;
-  return mlts_attn_bwd_dkdv_dma_workspace(s->B, s->Hq, s->Sq);  // lse2: B*Hq*Sq + 1 floats
+  return mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);  // lse2: B*Hq*Sq + 1 floats
 }
 
 int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   int rc;
-  int variant = dkdv_variant(D);
   // the newer kernels address rows of a tile with 32-bit element offsets
   const int64_t lim = int64_t{1} << 24;
-  if (p.qs[2] >= lim || p.ks[2] >= lim || p.vs[2] >= lim || bp.dos[2] >= lim) variant = 0;
-  if (variant == 2) {
+  const bool staged = use_staged_bwd() || p.qs[2] >= lim || p.ks[2] >= lim || p.vs[2] >= lim || bp.dos[2] >= lim;
+  if (!staged) {
     rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, workspace, st);
-  } else if (variant == 1) {
-    rc = mlts_attn_bwd_dkdv_bf16_dma(bp, mode, workspace, st);
   } else if (D == 128) {
     if (mode == MLTS_MASK_NONE) rc = launch_bwd<128, MLTS_MASK_NONE>(bp, st);
     else if (mode == MLTS_MASK_CAUSAL) rc = launch_bwd<128, MLTS_MASK_CAUSAL>(bp, st);
@@ -441,6 +434,6 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
-  if (variant == 2) return mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
+  if (!staged) return mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
   return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

@@ -156,7 +156,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     qt_begin = first_q <= 0 ? 0 : first_q / BQ;
   }
   const int span = qt_begin < nqt ? nqt - qt_begin : 0;
-  const int total_it = span * group;
 
   int4 kstats[2];
   if (MODE == MLTS_MASK_DOC) {
@@ -172,18 +171,29 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     kpos = p.k_pos[static_cast<int64_t>(b) * p.Sk + kj];
     kseq = p.k_seq[static_cast<int64_t>(b) * p.Sk + kj];
   }
-  auto block_needs = [&](int it) -> bool {
+  // The walk over (query head of the group, query tile) is kept as two counters; a position past the end has
+  // h == group.  (No division by the runtime tile count in the loop.)
+  struct Pos {
+    int qt, h;  // query tile relative to qt_begin, head within the GQA group
+  };
+  auto at_end = [&](const Pos& x) -> bool { return x.h >= group || span == 0; };
+  auto tile_needed = [&](const Pos& x) -> bool {
     if (MODE != MLTS_MASK_DOC) return true;
-    const int qt = qt_begin + it % span;
-    const int4 qs4 = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt];
+    const int4 qs4 = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt_begin + x.qt];
     return classify_doc_tile(qs4, kstats[0]) != TILE_SKIP || classify_doc_tile(qs4, kstats[1]) != TILE_SKIP;
   };
-  auto next_it = [&](int it) -> int {
-    while (it < total_it && !block_needs(it)) ++it;
-    return it;
+  auto step = [&](Pos& x) {
+    if (++x.qt == span) {
+      x.qt = 0;
+      ++x.h;
+    }
   };
-  auto classify = [&](int it) -> int {  // for this wavefront's 32 keys; identical in both roles of a key block
-    const int qt = qt_begin + it % span;
+  auto first_needed = [&](Pos x) -> Pos {  // x itself or the next position whose tile is needed
+    while (!at_end(x) && !tile_needed(x)) step(x);
+    return x;
+  };
+  auto classify = [&](const Pos& x) -> int {  // for this wavefront's 32 keys; identical in both roles of a key block
+    const int qt = qt_begin + x.qt;
     const int q0 = qt * BQ;
     int cls = TILE_FULL;
     if (MODE == MLTS_MASK_CAUSAL) {
@@ -220,9 +230,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   v4i32 stg_q[NLD], stg_d[NLD];
   float stg_s = 0.f;
   const uint32_t lds0_ = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
-  auto stage_load = [&](int it) {
-    const int hq = hkv * group + it / span;
-    const int q0 = (qt_begin + it % span) * BQ;
+  auto stage_load = [&](const Pos& x) {
+    const int hq = hkv * group + x.h;
+    const int q0 = (qt_begin + x.qt) * BQ;
     const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1] + static_cast<int64_t>(q0) * p.qs[2];
     const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1] + static_cast<int64_t>(q0) * bp.dos[2];
     const int last = p.Sq - 1 - q0;  // rows past the end repeat the last query; their lse2 is +inf
@@ -595,19 +605,21 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   // stored into stage (k + 1) % 3, which held tile k - 2 (role 1 finished it before this barrier). ----
   auto tile_loop = [&](auto role_tag) {
     constexpr int ROLE = decltype(role_tag)::value;
-    int it = next_it(0);
-    if (it < total_it) {
+    Pos it = first_needed(Pos{0, 0});
+    if (!at_end(it)) {
       stage_load(it);
       stage_store(0);
     }
     int stage = 0, k = 0;
     bool prev_active = false;
     int prev_stage = 0;
-    while (it < total_it) {
-      const int itn = next_it(it + 1);
+    while (!at_end(it)) {
+      Pos itn = it;
+      step(itn);
+      itn = first_needed(itn);
       drain_and_barrier();
-      if (itn < total_it) stage_load(itn);
-      const int q0 = (qt_begin + it % span) * BQ;
+      if (!at_end(itn)) stage_load(itn);
+      const int q0 = (qt_begin + it.qt) * BQ;
       const int cls = classify(it);
       const int pbuf = (k & 1) * (4 * PBUF_BYTES);
       if (ROLE == 0) {
@@ -620,7 +632,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         if (cls != TILE_SKIP) role1_dp(stage);
         if (prev_active) role1_dk(prev_stage);
       }
-      if (itn < total_it) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
+      if (!at_end(itn)) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
       prev_active = cls != TILE_SKIP;
       prev_stage = stage;
       it = itn;
@@ -686,6 +698,8 @@ int launch_mode(const AttnBwdParams& bp, int mode, const float* lse2, hipStream_
 }
 
 }  // namespace
+
+int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq) { return (((B * Hq * Sq + 1) * 4 + 255) / 256) * 256; }
 
 // head_dim 64 or 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
 int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
