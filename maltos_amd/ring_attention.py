@@ -9,6 +9,13 @@ Q/K/V chunk in zigzag layout and, ring step by ring step, the K/V chunk of rank 
 Block outputs are merged in fp32 with a log-sum-exp merge; the backward pass re-runs the same
 schedule with the GLOBAL out / LSE and accumulates dQ and the per-chunk dK/dV in fp32.
 
+Packed documents (sequence ids given) take the other path of the reference
+(_flash_packed_ring_forward/backward, functional.py:823-1009): every step attends all local queries to the whole
+arriving chunk under the document mask "same sequence id, not PAD, k_pos <= q_pos", with the positions and sequence
+ids travelling with the chunk.  The reference packs runs and key prefixes for flash_attn_varlen (flash_utils.py:
+566-962, a Python loop with host reads per run); here the kernels take the ids directly and skip the 64-key tiles
+no query can see, so there is no packing step and no host synchronisation.
+
 What moves K/V between ranks is a separate concern (the reference uses P2P send/recv): here it is
 the `kv_source` callable, which returns the chunk a step needs.  On one GPU the chunks are simply
 resident; nothing in this module touches torch.distributed.
@@ -93,6 +100,60 @@ class _ZigzagRingFunction(torch.autograd.Function):
         return (dq.to(q.dtype), None, None, *grads)
 
 
+class _PackedRingFunction(torch.autograd.Function):
+    """flat = (k, v, positions, sequence_ids) of rank 0, of rank 1, ...; ids are int [B, S_chunk]."""
+
+    @staticmethod
+    def forward(ctx, q: torch.Tensor, q_pos: torch.Tensor, q_seq: torch.Tensor, rank: int, world_size: int, *flat):
+        if len(flat) != 4 * world_size:
+            raise ValueError(f"expected {4 * world_size} chunk tensors, got {len(flat)}")
+        running_out = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+        for step in range(world_size):
+            k, v, k_pos, k_seq = flat[4 * ((rank - step) % world_size):][:4]
+            o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, q_pos=q_pos, k_pos=k_pos, q_seq=q_seq,
+                                           k_seq=k_seq)
+            ops.attention_merge_(running_out, running_lse, o, lse, 0)  # a block nobody sees into is (0, -inf)
+        out = running_out.to(dtype=flat[1].dtype)
+        ctx.save_for_backward(q, q_pos, q_seq, out, running_lse, *flat)
+        ctx.rank, ctx.world_size = rank, world_size
+        ctx.mark_non_differentiable(running_lse)
+        return out, running_lse
+
+    @staticmethod
+    def backward(ctx, dout: torch.Tensor, _dlse):
+        q, q_pos, q_seq, out, lse, *flat = ctx.saved_tensors
+        rank, world_size = ctx.rank, ctx.world_size
+        dout = dout.contiguous()
+        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        grads: list[torch.Tensor | None] = [None] * (4 * world_size)
+        for step in range(world_size):
+            src = (rank - step) % world_size
+            k, v, k_pos, k_seq = flat[4 * src:][:4]
+            dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
+            dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+            ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dk, dv, mask_mode=ops.MASK_DOC, q_pos=q_pos,
+                                              k_pos=k_pos, q_seq=q_seq, k_seq=k_seq)
+            grads[4 * src] = dk.to(k.dtype)
+            grads[4 * src + 1] = dv.to(v.dtype)
+        return (dq.to(q.dtype), None, None, None, None, *grads)
+
+
+def packed_ring_attention(q: torch.Tensor, kv_chunks: Sequence[KvChunk], *, q_positions: torch.Tensor,
+                          q_sequence_ids: torch.Tensor, kv_positions: Sequence[torch.Tensor],
+                          kv_sequence_ids: Sequence[torch.Tensor], rank: int, world_size: int, return_lse: bool = False):
+    """Rank `rank`'s attention output for packed documents: kv_chunks[r], kv_positions[r], kv_sequence_ids[r] describe
+    rank r's chunk ([batch, kv_heads, s_r, head_dim] and [batch, s_r]); q_positions / q_sequence_ids are this rank's.
+    Any token order inside a chunk (zigzag included) is fine: the mask is evaluated per (query, key) pair."""
+    if not (len(kv_chunks) == len(kv_positions) == len(kv_sequence_ids) == world_size):
+        raise ValueError(f"need K/V, positions and sequence ids for each of the {world_size} ranks")
+    flat: list[torch.Tensor] = []
+    for (k, v), pos, seq in zip(kv_chunks, kv_positions, kv_sequence_ids):
+        flat += [k, v, pos, seq]
+    out, lse = _PackedRingFunction.apply(q, q_positions, q_sequence_ids, rank, world_size, *flat)
+    return (out, lse) if return_lse else out
+
+
 def zigzag_ring_attention(q: torch.Tensor, kv_chunks: Sequence[KvChunk], *, rank: int, world_size: int,
                           return_lse: bool = False):
     """Rank `rank`'s attention output for its zigzag query chunk; kv_chunks[r] = (k, v) of rank r, each
@@ -111,19 +172,21 @@ class HipRingAttentionCore(nn.Module):
 
     With world_size == 1 it is plain local attention, as the reference's core is
     (runtime/layers/ring_attention.py:45-54).  With world_size > 1 the caller supplies
-    `kv_source(rank, k_local, v_local) -> [(k, v) for every rank]`, the seam where a transport plugs in.
+    `kv_source(rank, k_local, v_local) -> [(k, v) for every rank]`, the seam where a transport plugs in, and for
+    packed documents `meta_source(rank, positions_local, sequence_ids_local) -> [(positions, sequence_ids) ...]`.
     """
 
     preserves_native_gqa = True
 
     def __init__(self, *, rank: int = 0, world_size: int = 1,
                  kv_source: Callable[[int, torch.Tensor, torch.Tensor], Sequence[KvChunk]] | None = None,
+                 meta_source: Callable[[int, torch.Tensor, torch.Tensor], Sequence[KvChunk]] | None = None,
                  attention_backend: str = AttentionBackend.HIP) -> None:
         super().__init__()
         self.attention_backend = validate_attention_backend(attention_backend)
         if world_size > 1 and kv_source is None:
             raise ValueError("HipRingAttentionCore with world_size > 1 needs a kv_source")
-        self.rank, self.world_size, self.kv_source = rank, world_size, kv_source
+        self.rank, self.world_size, self.kv_source, self.meta_source = rank, world_size, kv_source, meta_source
 
     def forward(self, q, k, v, position_offset: int, position_ids=None, sequence_ids=None) -> torch.Tensor:
         if self.world_size == 1:
@@ -134,6 +197,15 @@ class HipRingAttentionCore(nn.Module):
                                     q_positions=positions, k_positions=positions, q_sequence_ids=sequences,
                                     k_sequence_ids=sequences)
         if sequence_ids is not None:
-            raise NotImplementedError("packed-document ring attention (varlen-prefix blocks) is not built yet")
+            if self.meta_source is None:
+                raise ValueError("packed-document ring attention needs a meta_source for the chunks' positions and ids")
+            positions = canonical_position_ids(position_ids, batch_size=q.size(0), seq_len=q.size(-2),
+                                               position_offset=position_offset, device=q.device)
+            sequences = canonical_sequence_ids(sequence_ids, batch_size=q.size(0), seq_len=q.size(-2), device=q.device)
+            chunks = self.kv_source(self.rank, k, v)
+            meta = self.meta_source(self.rank, positions, sequences)
+            return packed_ring_attention(q, chunks, q_positions=positions, q_sequence_ids=sequences,
+                                         kv_positions=[m[0] for m in meta], kv_sequence_ids=[m[1] for m in meta],
+                                         rank=self.rank, world_size=self.world_size)
         chunks = self.kv_source(self.rank, k, v)
         return zigzag_ring_attention(q, chunks, rank=self.rank, world_size=self.world_size)

@@ -218,6 +218,38 @@ def zigzag_ring_backward(dout, q, kv_chunks, out, lse, *, rank: int, world_size:
     return dq, dkv
 
 
+# ---- runtime/layers/functional.py:823-897 -------------------------------------------------------
+def packed_ring_forward(q, kv_chunks, q_pos, q_seq, meta_chunks, *, rank: int, world_size: int):
+    """One rank's forward for packed documents: at ring step s the K/V chunk of rank (rank - s) mod W arrives with
+    its positions and sequence ids; a query sees the keys of its own document with k_pos <= q_pos (the varlen
+    prefix blocks of flash_utils.py:566-962 select exactly those); blocks with no visible key merge as (0, -inf).
+    kv_chunks[r] = (k, v), meta_chunks[r] = (positions, sequence_ids) of rank r."""
+    running_out = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+    running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+    for step in range(world_size):
+        src = (rank - step) % world_size
+        k, v = kv_chunks[src]
+        k_pos, k_seq = meta_chunks[src]
+        o, l = attention_with_lse(q, k, v, doc_mask(q_pos, k_pos, q_seq, k_seq))
+        running_out, running_lse = merge_attention_blocks(running_out, running_lse, o, l)
+    return running_out.to(kv_chunks[rank][1].dtype), running_lse
+
+
+# ---- runtime/layers/functional.py:900-1009 ------------------------------------------------------
+def packed_ring_backward(dout, q, kv_chunks, q_pos, q_seq, meta_chunks, out, lse, *, rank: int, world_size: int):
+    """dq (fp32) and this rank's contribution to every chunk's dk/dv (fp32), global out/lse in each block."""
+    dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+    dkv = {}
+    for step in range(world_size):
+        src = (rank - step) % world_size
+        k, v = kv_chunks[src]
+        k_pos, k_seq = meta_chunks[src]
+        bdq, bdk, bdv = attention_backward_explicit(dout, q, k, v, out, lse, doc_mask(q_pos, k_pos, q_seq, k_seq))
+        dq += bdq
+        dkv[src] = (bdk.float(), bdv.float())
+    return dq, dkv
+
+
 # ---- runtime/layers/ring_attention.py:221-258 (eager online softmax, single step form) ----------
 def online_softmax_update(q, k, v, mask, running_max, running_sum, running_acc, *, scale: float | None = None):
     """(running_max, running_sum, running_acc) update in fp32; final output is acc / sum.clamp_min(1e-20)."""

@@ -9,7 +9,8 @@ Tolerances
                       bf16 ulp of the expected value, the rounding any bf16 output carries (it matters only
                       for |want| > ~5, e.g. dV rows that sum many queries).
       LSE (fp32)    : 2e-3 absolute.
-  * reference ring test vectors (fp32, head_dim 3): forward 1e-5, backward 2e-5, the reference's own bars.
+  * reference ring test vectors (fp32, head_dim 3): forward 1e-5, backward 2e-5, the reference's own bars
+    (zigzag ring and packed-document ring).
 """
 import pytest
 import torch
@@ -19,7 +20,7 @@ from maltos_amd.attention_backend import causal_attention
 from maltos_amd.flash_utils import (flash_attn_dense, flash_attn_dense_backward, flash_attn_dense_with_lse,
                                     flash_attn_varlen)
 from maltos_amd.llama import HipAttentionCore
-from maltos_amd.ring_attention import HipRingAttentionCore, zigzag_ring_attention
+from maltos_amd.ring_attention import HipRingAttentionCore, packed_ring_attention, zigzag_ring_attention
 from maltos_amd.ring_layout import expected_zigzag_ring_positions
 from oracle import attention as oa
 
@@ -297,3 +298,71 @@ def test_zigzag_ring_bf16_matches_global_causal(dev):
     solo = HipRingAttentionCore()(all_q[:, :, :256].to(dev), all_k[:, :, :256].to(dev), all_v[:, :, :256].to(dev), 0)
     want, _ = oa.attention_with_lse(all_q[:, :, :256], all_k[:, :, :256], all_v[:, :, :256], oa.causal_mask(256, 256, "cpu"))
     check(solo, want, torch.bfloat16, "single-rank ring")
+
+
+def test_packed_ring_reference_scenario_fp32(dev, known_answers):
+    """tests/sequence_ids_attention_mask.py:366-434 of the reference: two documents and a PAD token in zigzag order over
+    two ranks; every rank's merged output equals global document-masked attention at its tokens."""
+    spec = known_answers["packed_ring"]
+    w, s_loc, total = spec["world_size"], spec["local_seq_len"], spec["local_seq_len"] * spec["world_size"]
+    mk = lambda seed: torch.randn((spec["batch"], spec["heads"], total, spec["head_dim"]), generator=torch.Generator().manual_seed(seed))
+    all_q, all_k, all_v = (mk(spec["seeds"][n]) for n in "qkv")
+    all_pos = torch.tensor(spec["positions"]).view(1, total)
+    all_seq = torch.tensor(spec["sequence_ids"]).view(1, total)
+    idx = [expected_zigzag_ring_positions(s_loc, rank=r, world_size=w, device=torch.device("cpu")) for r in range(w)]
+    gq, gk, gv = (t.clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, glse = oa.attention_with_lse(gq, gk, gv, oa.doc_mask(all_pos, all_pos, all_seq, all_seq))
+    dout_all = torch.randn(gout.shape, generator=torch.Generator().manual_seed(5))
+    gout.backward(dout_all)
+    dk_sum, dv_sum = torch.zeros_like(all_k), torch.zeros_like(all_v)
+    pc = [all_pos.index_select(1, i).to(dev) for i in idx]
+    sc = [all_seq.index_select(1, i).to(dev) for i in idx]
+    for rank in range(w):
+        q = all_q.index_select(2, idx[rank]).to(dev).requires_grad_(True)
+        chunks = [(all_k.index_select(2, i).to(dev).requires_grad_(True), all_v.index_select(2, i).to(dev).requires_grad_(True)) for i in idx]
+        out, lse = packed_ring_attention(q, chunks, q_positions=pc[rank], q_sequence_ids=sc[rank], kv_positions=pc,
+                                         kv_sequence_ids=sc, rank=rank, world_size=w, return_lse=True)
+        assert torch.allclose(out.cpu(), gout.detach().index_select(2, idx[rank]), atol=spec["forward_atol"])
+        want_lse = glse.index_select(2, idx[rank])
+        fin = torch.isfinite(want_lse)
+        assert torch.equal(torch.isfinite(lse.cpu()), fin)
+        assert torch.allclose(lse.cpu()[fin], want_lse[fin], atol=spec["forward_atol"])
+        out.backward(dout_all.index_select(2, idx[rank]).to(dev))
+        assert torch.allclose(q.grad.cpu(), gq.grad.index_select(2, idx[rank]), atol=2e-5)
+        for src, (k, v) in enumerate(chunks):
+            dk_sum.index_add_(2, idx[src], k.grad.cpu())
+            dv_sum.index_add_(2, idx[src], v.grad.cpu())
+    assert torch.allclose(dk_sum, gk.grad, atol=2e-5)
+    assert torch.allclose(dv_sum, gv.grad, atol=2e-5)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_packed_ring_bf16_matches_global_document_attention(dev, D):
+    world_size, s_loc, B, Hq, Hkv = 4, 256, 2, 4, 2
+    total = world_size * s_loc
+    gen = torch.Generator().manual_seed(40 + D)
+    all_q, all_k, all_v = bshd(B, Hq, total, D, gen, torch.bfloat16), bshd(B, Hkv, total, D, gen, torch.bfloat16), bshd(B, Hkv, total, D, gen, torch.bfloat16)
+    all_pos, all_seq = make_docs(B, total, gen, 400, pad_tail=37)
+    idx = [expected_zigzag_ring_positions(s_loc, rank=r, world_size=world_size, device=torch.device("cpu")) for r in range(world_size)]
+    gq, gk, gv = (t.detach().float().clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, _ = oa.attention_with_lse(gq, gk, gv, oa.doc_mask(all_pos, all_pos, all_seq, all_seq))
+    dout_all = torch.randn(gout.shape, generator=gen).bfloat16()
+    gout.backward(dout_all.float())
+    dk_sum, dv_sum = torch.zeros_like(gk.grad), torch.zeros_like(gv.grad)
+    pc = [all_pos.index_select(1, i).to(dev) for i in idx]
+    sc = [all_seq.index_select(1, i).to(dev) for i in idx]
+    for rank in range(world_size):
+        q = all_q.index_select(2, idx[rank]).to(dev).requires_grad_(True)
+        chunks = [(all_k.index_select(2, i).to(dev).requires_grad_(True), all_v.index_select(2, i).to(dev).requires_grad_(True)) for i in idx]
+        core = HipRingAttentionCore(rank=rank, world_size=world_size, kv_source=lambda r, k, v, c=chunks: c,
+                                    meta_source=lambda r, p, s: list(zip(pc, sc)))
+        out = core(q, chunks[rank][0], chunks[rank][1], 0, pc[rank], sc[rank])
+        check(out, gout.detach().index_select(2, idx[rank]), torch.bfloat16, f"packed ring O rank{rank}")
+        out.backward(dout_all.index_select(2, idx[rank]).to(dev))
+        check(q.grad, gq.grad.index_select(2, idx[rank]), torch.bfloat16, f"packed ring dQ rank{rank}")
+        for src, (k, v) in enumerate(chunks):
+            dk_sum.index_add_(2, idx[src], k.grad.float().cpu())
+            dv_sum.index_add_(2, idx[src], v.grad.float().cpu())
+    # each chunk's dK/dV is the sum of four bf16-rounded rank contributions
+    assert ((dk_sum - gk.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gk.grad.abs())).all()
+    assert ((dv_sum - gv.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gv.grad.abs())).all()

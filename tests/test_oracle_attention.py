@@ -193,6 +193,55 @@ def test_zigzag_ring_backward_invariant(known_answers, world_size):
     assert torch.allclose(dv_sum, gv.grad, atol=spec["backward_atol"])
 
 
+def _packed_ring_setup(spec):
+    """The reference's packed-ring scenario: two documents and a PAD token, spread over the ranks in zigzag order."""
+    b, h, s_loc, d, w = spec["batch"], spec["heads"], spec["local_seq_len"], spec["head_dim"], spec["world_size"]
+    total = s_loc * w
+    mk = lambda seed: torch.randn((b, h, total, d), generator=torch.Generator().manual_seed(seed))
+    all_q, all_k, all_v = (mk(spec["seeds"][n]) for n in "qkv")
+    all_pos = torch.tensor(spec["positions"]).view(1, total).expand(b, total)
+    all_seq = torch.tensor(spec["sequence_ids"]).view(1, total).expand(b, total)
+    idx = [oa.zigzag_positions(s_loc, rank=r, world_size=w) for r in range(w)]
+    pick = lambda t, dim: [t.index_select(dim, i) for i in idx]
+    return all_q, all_k, all_v, all_pos, all_seq, idx, pick
+
+
+def test_packed_ring_equals_global_document_attention(known_answers):
+    spec = known_answers["packed_ring"]
+    w = spec["world_size"]
+    all_q, all_k, all_v, all_pos, all_seq, idx, pick = _packed_ring_setup(spec)
+    qc, kc, vc, pc, sc = pick(all_q, 2), pick(all_k, 2), pick(all_v, 2), pick(all_pos, 1), pick(all_seq, 1)
+    gq, gk, gv = (t.clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, glse = oa.attention_with_lse(gq, gk, gv, oa.doc_mask(all_pos, all_pos, all_seq, all_seq))
+    # brute force of the rule the reference's test states, independent of doc_mask
+    for i in range(all_q.size(2)):
+        vis = [j for j in range(all_q.size(2)) if spec["sequence_ids"][i] >= 0
+               and spec["sequence_ids"][j] == spec["sequence_ids"][i] and spec["positions"][j] <= spec["positions"][i]]
+        if not vis:
+            assert gout[0, 0, i].abs().max() == 0
+            continue
+        p = torch.softmax(all_q[0, 0, i] @ all_k[0, 0, vis].T * all_q.size(-1) ** -0.5, dim=-1)
+        assert torch.allclose(gout[0, 0, i], p @ all_v[0, 0, vis], atol=1e-6)
+    dout_all = torch.randn(gout.shape, generator=torch.Generator().manual_seed(5))
+    gout.backward(dout_all)
+    dk_sum, dv_sum = torch.zeros_like(all_k), torch.zeros_like(all_v)
+    for rank in range(w):
+        out, lse = oa.packed_ring_forward(qc[rank], list(zip(kc, vc)), pc[rank], sc[rank], list(zip(pc, sc)), rank=rank,
+                                          world_size=w)
+        assert torch.allclose(out, gout.detach().index_select(2, idx[rank]), atol=spec["forward_atol"])
+        want_lse = glse.index_select(2, idx[rank])
+        assert torch.equal(torch.isfinite(lse), torch.isfinite(want_lse))
+        assert torch.allclose(lse[torch.isfinite(lse)], want_lse[torch.isfinite(lse)], atol=spec["forward_atol"])
+        dq, dkv = oa.packed_ring_backward(dout_all.index_select(2, idx[rank]), qc[rank], list(zip(kc, vc)), pc[rank],
+                                          sc[rank], list(zip(pc, sc)), out, lse, rank=rank, world_size=w)
+        assert torch.allclose(dq, gq.grad.index_select(2, idx[rank]), atol=2e-5)
+        for src, (dk, dv) in dkv.items():
+            dk_sum.index_add_(2, idx[src], dk)
+            dv_sum.index_add_(2, idx[src], dv)
+    assert torch.allclose(dk_sum, gk.grad, atol=2e-5)
+    assert torch.allclose(dv_sum, gv.grad, atol=2e-5)
+
+
 def test_online_softmax_equals_attention():
     g = torch.Generator().manual_seed(21)
     q = torch.randn(1, 2, 5, 8, generator=g)
