@@ -382,8 +382,32 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     }
   }
 
-  if (qrow < p.Sq) {
-    const float oscale = -p.scale;  // the accumulator holds K^T (-dS^T)
+  const float oscale = -p.scale;  // the accumulator holds K^T (-dS^T)
+  const bool rows16 = ((bp.dqs[0] | bp.dqs[1] | bp.dqs[2]) & 7) == 0 && (reinterpret_cast<uintptr_t>(bp.dq_acc) & 15) == 0;
+  if (!bp.accumulate_f32 && rows16) {
+    // bf16 rows through LDS (each wavefront owns 32 rows x RB bytes, tile-row swizzle), so that global stores are
+    // 16 bytes per lane and cover whole rows
+    drain_and_barrier();  // every wavefront has finished reading the last K/V tile
+    unsigned char* ebase = smem + wave * (32 * RB);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(dqacc[db][g * 4 + r] * oscale);
+        *reinterpret_cast<bf16x4*>(ebase + l32 * RB + (((db * 4 + g) ^ swz<D>(l32 & 15)) << 4) + hh * 8) = w;
+      }
+    }
+    bf16_t* obase = reinterpret_cast<bf16_t*>(bp.dq_acc) + b * bp.dqs[0] + hq * bp.dqs[1];
+#pragma unroll
+    for (int i = 0; i < 32 * CPR / 64; ++i) {
+      const int idx = i * 64 + lane;
+      const int row = idx / CPR, chunk = idx % CPR;
+      const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ swz<D>(row & 15)) << 4));
+      if (wq0 + row < p.Sq) *reinterpret_cast<v4i32*>(obase + static_cast<int64_t>(wq0 + row) * bp.dqs[2] + chunk * 8) = x;
+    }
+  } else if (qrow < p.Sq) {
     const int64_t rowoff = b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(qrow) * bp.dqs[2];
 #pragma unroll
     for (int db = 0; db < DB; ++db) {

@@ -133,18 +133,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   const int kj = wkv0 + l32;
 
   // ---- this wavefront's stationary operand (B operand of its first GEMM): K for role 0, -V for role 1 ----
-  bf16x8 kvf[KS];
+  // (loaded here, sign applied after the first tile's loads have been issued too: one memory latency, not two)
+  v4i32 kvraw[KS];
   {
     const bf16_t* src = role == 0 ? static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1] + static_cast<int64_t>(kj) * p.ks[2]
                                   : static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1] + static_cast<int64_t>(kj) * p.vs[2];
-    const int flip = role == 0 ? 0 : static_cast<int>(0x80008000u);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      v4i32 x = {0, 0, 0, 0};
-      if (kj < p.Sk) x = *reinterpret_cast<const v4i32*>(src + ks * 16 + hh * 8);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] ^= flip;
-      kvf[ks] = as_frag(x);
+      kvraw[ks] = v4i32{0, 0, 0, 0};
+      if (kj < p.Sk) kvraw[ks] = *reinterpret_cast<const v4i32*>(src + ks * 16 + hh * 8);
     }
   }
 
@@ -265,6 +262,19 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     if (tid < 2 * BQ)
       asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(lds0_ + stage * STAGE_BYTES + tid * 4), "v"(stg_s), "n"(STAT_OFF));
   };
+
+  const Pos it0 = first_needed(Pos{0, 0});
+  if (!at_end(it0)) stage_load(it0);
+  bf16x8 kvf[KS];
+  {
+    const int flip = role == 0 ? 0 : static_cast<int>(0x80008000u);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) kvraw[ks][i] ^= flip;
+      kvf[ks] = as_frag(kvraw[ks]);
+    }
+  }
 
   // ---- per-lane LDS offsets (tile invariant) ----
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
@@ -603,13 +613,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   // ---- tile loop, one instance per role (so that the state of one role is not live in the other's code).
   // Barrier k: tile k is in LDS and role 0 has handed over P of tile k - 1.  Tile k + 1 is fetched behind it and
   // stored into stage (k + 1) % 3, which held tile k - 2 (role 1 finished it before this barrier). ----
+  int last_stage = 0;  // the only stage that role 1 still reads after the last barrier
   auto tile_loop = [&](auto role_tag) {
     constexpr int ROLE = decltype(role_tag)::value;
-    Pos it = first_needed(Pos{0, 0});
-    if (!at_end(it)) {
-      stage_load(it);
-      stage_store(0);
-    }
+    Pos it = it0;  // its loads were issued in the prologue
+    if (!at_end(it)) stage_store(0);
     int stage = 0, k = 0;
     bool prev_active = false;
     int prev_stage = 0;
@@ -644,6 +652,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       role1_ds(((k - 1) & 1) * (4 * PBUF_BYTES));
       role1_dk(prev_stage);
     }
+    last_stage = prev_stage;
   };
   if (role == 0) tile_loop(std::integral_constant<int, 0>{});
   else tile_loop(std::integral_constant<int, 1>{});
@@ -652,17 +661,46 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   {
     const float oscale = role == 0 ? 1.0f : -p.scale;  // role 1 holds -dS^T Q
     void* optr = role == 0 ? bp.dv : bp.dk;
-    const int64_t* os = role == 0 ? bp.dvs : bp.dks;
+    const int64_t os[3] = {role == 0 ? bp.dvs[0] : bp.dks[0], role == 0 ? bp.dvs[1] : bp.dks[1], role == 0 ? bp.dvs[2] : bp.dks[2]};
+    const bool rows16 = ((os[0] | os[1] | os[2]) & 7) == 0 && (reinterpret_cast<uintptr_t>(optr) & 15) == 0;
+    if (!bp.accumulate_f32 && rows16) {
+      // bf16 rows through LDS, so that global stores are 16 bytes per lane and cover whole rows: each wavefront owns
+      // 32 rows x RB bytes of a stage that nobody reads any more (role 0: last_stage + 1, role 1: last_stage + 2);
+      // chunk ^ (4 if row & 4) keeps the two half-wavefronts (rows 4 apart) on different banks
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      int es = last_stage + 1 + role;
+      es = es >= STAGES ? es - STAGES : es;
+      unsigned char* ebase = smem + es * STAGE_BYTES + kb * (32 * RB);
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int d = db * 32 + l32;
+      for (int db = 0; db < DB; ++db) {
+        const int col = db * 32 + l32;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
-        if (row < p.Sk) {
-          const int64_t o = b * os[0] + hkv * os[1] + static_cast<int64_t>(row) * os[2] + d;
-          if (bp.accumulate_f32) static_cast<float*>(optr)[o] += acc[db][e] * oscale;
-          else static_cast<bf16_t*>(optr)[o] = static_cast<bf16_t>(acc[db][e] * oscale);
+        for (int e = 0; e < 16; ++e) {
+          const int row = (e >> 2) * 8 + hh * 4 + (e & 3);
+          const int chunk = (col >> 3) ^ (((row >> 2) & 1) << 2);
+          *reinterpret_cast<bf16_t*>(ebase + row * RB + chunk * 16 + (col & 7) * 2) = static_cast<bf16_t>(acc[db][e] * oscale);
+        }
+      }
+      bf16_t* obase = static_cast<bf16_t*>(optr) + b * os[0] + hkv * os[1];
+#pragma unroll
+      for (int i = 0; i < 32 * CPR / 64; ++i) {
+        const int idx = i * 64 + lane;
+        const int row = idx / CPR, chunk = idx % CPR;
+        const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ (((row >> 2) & 1) << 2)) << 4));
+        if (wkv0 + row < p.Sk) *reinterpret_cast<v4i32*>(obase + static_cast<int64_t>(wkv0 + row) * os[2] + chunk * 8) = x;
+      }
+    } else {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = db * 32 + l32;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
+          if (row < p.Sk) {
+            const int64_t o = b * os[0] + hkv * os[1] + static_cast<int64_t>(row) * os[2] + d;
+            if (bp.accumulate_f32) static_cast<float*>(optr)[o] += acc[db][e] * oscale;
+            else static_cast<bf16_t*>(optr)[o] = static_cast<bf16_t>(acc[db][e] * oscale);
+          }
         }
       }
     }

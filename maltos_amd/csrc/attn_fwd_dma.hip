@@ -427,11 +427,34 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  if (qrow < p.Sq) {
-    if (hh == 0) {
-      p.lse[(static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow] =
-          l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+  if (qrow < p.Sq && hh == 0) {
+    p.lse[(static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow] =
+        l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+  }
+  const bool rows16 = ((p.os[0] | p.os[1] | p.os[2]) & 7) == 0 && (reinterpret_cast<uintptr_t>(p.o) & 15) == 0;
+  if (rows16) {
+    // rows through LDS (each wavefront owns 32 rows x RB bytes, tile-row swizzle), so that global stores are 16 bytes
+    // per lane and cover whole rows
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // nobody reads a K/V tile any more
+    unsigned char* ebase = smem + wave * (32 * RB);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        bf16x4 w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(oacc[db][g * 4 + r] * inv);
+        *reinterpret_cast<bf16x4*>(ebase + l32 * RB + (((db * 4 + g) ^ swz<D>(l32 & 15)) << 4) + hh * 8) = w;
+      }
     }
+#pragma unroll
+    for (int i = 0; i < 32 * CPR / 64; ++i) {
+      const int idx = i * 64 + lane;
+      const int row = idx / CPR, chunk = idx % CPR;
+      const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ swz<D>(row & 15)) << 4));
+      if (wq0 + row < p.Sq) *reinterpret_cast<v4i32*>(O + static_cast<int64_t>(wq0 + row) * p.os[2] + chunk * 8) = x;
+    }
+  } else if (qrow < p.Sq) {
     bf16_t* orow = O + static_cast<int64_t>(qrow) * p.os[2];
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
