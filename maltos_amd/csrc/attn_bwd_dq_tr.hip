@@ -171,8 +171,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   // ---- tile loader: 64 bytes per thread, chunks t and t + 512 of the K tile and of the V tile (chunk c = row c/16,
   // stored 16-byte slot c%16, source slot (c%16) ^ swz(row)); registers now, ds_write_b128 after this tile's work ----
-  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
-  // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
+  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread byte offset that is the same for every tile
+  // not cut by the end of the sequence (a byte offset; row strides below 2^24 elements, checked by the caller)
   int ld_row[NLD], ld_col[NLD];
   uint32_t ld_koff[NLD], ld_voff[NLD];
 #pragma unroll
@@ -180,8 +180,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     const int c = tid + n * THREADS;
     ld_row[n] = c / CPR;
     ld_col[n] = ((c % CPR) ^ swz<D>((c / CPR) & 15)) * 8;
-    ld_koff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.ks[2]) + ld_col[n];
-    ld_voff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n];
+    ld_koff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.ks[2]) + ld_col[n]) * 2;  // bytes
+    ld_voff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n]) * 2;
   }
   v4i32 stg_k[NLD], stg_v[NLD];
   auto stage_load = [&](int j) {
@@ -194,11 +194,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       uint32_t ko = ld_koff[n], vo = ld_voff[n];
       if (last < BN - 1) {
         const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
-        ko = r * static_cast<uint32_t>(p.ks[2]) + ld_col[n];
-        vo = r * static_cast<uint32_t>(p.vs[2]) + ld_col[n];
+        ko = (r * static_cast<uint32_t>(p.ks[2]) + ld_col[n]) * 2;
+        vo = (r * static_cast<uint32_t>(p.vs[2]) + ld_col[n]) * 2;
       }
-      stg_k[n] = *reinterpret_cast<const v4i32*>(Kt + ko);
-      stg_v[n] = *reinterpret_cast<const v4i32*>(Vt + vo);
+      stg_k[n] = *reinterpret_cast<const v4i32*>(reinterpret_cast<const char*>(Kt) + ko);
+      stg_v[n] = *reinterpret_cast<const v4i32*>(reinterpret_cast<const char*>(Vt) + vo);
     }
   };
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   // c % CPR, source slot (c % CPR) ^ swz(row)) and written to LDS with ds_write_b128 after this tile's work.  Threads 0..127 also
   // carry the 64 + 64 row statistics (lse2, delta). ----
   const int64_t lse2_inf = static_cast<int64_t>(p.B) * p.Hq * p.Sq;  // index of the +inf entry
-  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread element offset that is the same for every tile
+  // addresses: a wave-uniform tile pointer plus a 32-bit per-thread byte offset that is the same for every tile
   // not cut by the end of the sequence (row strides below 2^24 elements, checked by the caller)
   int ld_row[NLD], ld_col[NLD];
   uint32_t ld_qoff[NLD], ld_doff[NLD];
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     const int c = tid + n * THREADS;
     ld_row[n] = c / CPR;
     ld_col[n] = ((c % CPR) ^ swz<D>((c / CPR) & 15)) * 8;
-    ld_qoff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.qs[2]) + ld_col[n];
-    ld_doff[n] = static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(bp.dos[2]) + ld_col[n];
+    ld_qoff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.qs[2]) + ld_col[n]) * 2;  // bytes
+    ld_doff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(bp.dos[2]) + ld_col[n]) * 2;
   }
   v4i32 stg_q[NLD], stg_d[NLD];
   float stg_s = 0.f;
@@ -238,11 +238,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       uint32_t qo = ld_qoff[n], dofs = ld_doff[n];
       if (last < BQ - 1) {
         const uint32_t r = static_cast<uint32_t>(min(ld_row[n], last));
-        qo = r * static_cast<uint32_t>(p.qs[2]) + ld_col[n];
-        dofs = r * static_cast<uint32_t>(bp.dos[2]) + ld_col[n];
+        qo = (r * static_cast<uint32_t>(p.qs[2]) + ld_col[n]) * 2;
+        dofs = (r * static_cast<uint32_t>(bp.dos[2]) + ld_col[n]) * 2;
       }
-      stg_q[n] = *reinterpret_cast<const v4i32*>(Q + qo);
-      stg_d[n] = *reinterpret_cast<const v4i32*>(dO + dofs);
+      stg_q[n] = *reinterpret_cast<const v4i32*>(reinterpret_cast<const char*>(Q) + qo);
+      stg_d[n] = *reinterpret_cast<const v4i32*>(reinterpret_cast<const char*>(dO) + dofs);
     }
     if (tid < 2 * BQ) {
       const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
