@@ -29,7 +29,8 @@ struct DqCfg {
   static constexpr int CPR = RB / 16;                  // 16-byte chunks per row
   static constexpr int TILE_BYTES = BN * RB;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int PRO_BYTES = 2 * BM * RB;        // the prologue passes the Q and dO tiles through LDS
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES > PRO_BYTES ? STAGES * STAGE_BYTES : PRO_BYTES;
   static constexpr int NLD = BN * CPR / THREADS;       // 16-byte chunks per thread and tile (2 or 1)
 };
 
@@ -112,24 +113,26 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
 
-  bf16x8 qf[KS], ndof[KS];  // Q and -dO fragments (B operands)
+  // Prologue loads, all issued before the first use of any of them.  The Q and dO tiles are fetched with whole-row
+  // 16-byte loads (chunk c = tid + 512 n: row c / CPR, stored slot c % CPR, source slot (c % CPR) ^ swz(row), the tile
+  // layout) and handed to the wavefronts through LDS: a fragment load straight from global memory touches 32 rows per
+  // instruction and was measured at ~90 cycles per instruction, 8 us for the workgroup.  Rows past the end repeat
+  // the last query (their lse2 is +inf, so they contribute nothing and are never stored).
+  constexpr int NPRO = BM * CPR / THREADS;
+  v4i32 pro_q[NPRO], pro_d[NPRO];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    v4i32 a = {0, 0, 0, 0}, c = {0, 0, 0, 0};
-    if (qrow < p.Sq) {
-      a = *reinterpret_cast<const v4i32*>(Q + static_cast<int64_t>(qrow) * p.qs[2] + ks * 16 + hh * 8);
-      c = *reinterpret_cast<const v4i32*>(dO + static_cast<int64_t>(qrow) * bp.dos[2] + ks * 16 + hh * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) c[i] ^= static_cast<int>(0x80008000u);
-    qf[ks] = as_frag(a);
-    ndof[ks] = as_frag(c);
+  for (int n = 0; n < NPRO; ++n) {
+    const int c = tid + n * THREADS;
+    const int row = c / CPR;
+    const int col = ((c % CPR) ^ swz<D>(row & 15)) * 8;
+    const int64_t r = min(q0 + row, p.Sq - 1);
+    pro_q[n] = *reinterpret_cast<const v4i32*>(Q + r * p.qs[2] + col);
+    pro_d[n] = *reinterpret_cast<const v4i32*>(dO + r * bp.dos[2] + col);
   }
-  float lse2 = INFINITY, delta = 0.f;  // +inf makes exp2(s - lse2) = 0 for rows that saw no key or lie past Sq
+  float lse_raw = -INFINITY, delta = 0.f;
   if (qrow < p.Sq) {
     const int64_t off = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow;
-    const float l = p.lse[off];
-    lse2 = l == -INFINITY ? INFINITY : l * kLog2e;
+    lse_raw = p.lse[off];
     delta = bp.delta[off];
   }
   int qpos = 0, qseq = -1;
@@ -212,6 +215,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     }
   };
 
+  const int j0 = next_tile(0);
+  if (j0 < j_end) stage_load(j0);
+
   // ---- per-lane LDS read offsets (tile invariant) ----
   // (LDS addresses of stage 0; the stage, the key block and the tile are added as instruction offsets)
   uint32_t ra[KS];  // row-major fragment (A operand): row l32 (+32 kb), chunk 2 ks + hh
@@ -227,6 +233,35 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       ta[part][db] = lds0 + rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
     }
   }
+
+  bf16x8 qf[KS], ndof[KS];  // Q and -dO fragments (B operands): row 32 wave + l32, the row-major fragment pattern
+  {
+    const uint32_t wbase = lds0 + tid * 16;
+#pragma unroll
+    for (int n = 0; n < NPRO; ++n) {
+      lds_write_b128<0>(wbase + n * (THREADS * 16), pro_q[n]);
+      lds_write_b128<0>(wbase + BM * RB + n * (THREADS * 16), pro_d[n]);
+    }
+    drain_and_barrier();
+    v4i32 fq[KS], fd[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      fq[ks] = lds_read_b128<0>(ra[ks] + wave * (32 * RB));
+      fd[ks] = lds_read_b128<0>(ra[ks] + wave * (32 * RB) + BM * RB);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      // (the registers are operands of the wait, so that the compiler cannot touch them before it)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fq[ks]), "+v"(fd[ks])::"memory");
+#pragma unroll
+      for (int i = 0; i < 4; ++i) fd[ks][i] ^= static_cast<int>(0x80008000u);
+      qf[ks] = as_frag(fq[ks]);
+      ndof[ks] = as_frag(fd[ks]);
+    }
+    drain_and_barrier();  // the K/V tiles may overwrite the Q and dO tiles from here on
+  }
+  // +inf makes exp2(s - lse2) = 0 for rows that saw no key or lie past Sq
+  const float lse2 = lse_raw == -INFINITY ? INFINITY : lse_raw * kLog2e;
 
   f32x16 dqacc[DB];  // -dQ^T / scale: register e <-> head-dim 32 db + 8 (e/4) + 4 hh + e%4, lane -> query row
 #pragma unroll
@@ -353,11 +388,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   // other stage (read last during tile k - 1) after the work on tile k.  There is one instance of the tile body
   // (with several, the register allocator keeps the dQ accumulators twice); masking is a branch inside it. ----
   {
-    int j = next_tile(0);
-    if (j < j_end) {
-      stage_load(j);
-      stage_store(0);
-    }
+    int j = j0;  // its loads were issued in the prologue
+    if (j < j_end) stage_store(0);
     int stage = 0;
     while (j < j_end) {
       const int jn = next_tile(j + 1);
