@@ -79,14 +79,18 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup):
     torch.cuda.synchronize()
     sec = (time.perf_counter() - t0) / steps
     kernels = {}
-    for name in ("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"):
+    for name in ("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq", "attn_bwd_dq_ds"):
         total_ms, launches = _lib.kernel_time_ms(name)
         if launches:
             kernels[name] = {"ms": total_ms / launches, "launches_per_step": launches / steps}
     _lib.kernel_timing(False)
-    # algorithmic flops per launch of each kernel (FlashAttention convention: 2 GEMMs forward, 5 backward)
+    # algorithmic flops per launch of each kernel (FlashAttention convention: 2 GEMMs forward, 5 backward: S, dP, dV,
+    # dK, dQ, each fwd_flops / 2)
     kernel_flops = {"attn_fwd": fwd_flops}
-    if "attn_bwd_dq" in kernels:  # split backward: dK/dV kernel carries 4 of the 5 GEMM-equivalents' share
+    if "attn_bwd_dq_ds" in kernels:  # dK/dV kernel hands dS over: it runs S, dP, dV, dK, the dQ kernel only dQ
+        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops * 0.8
+        kernel_flops["attn_bwd_dq_ds"] = 2.5 * fwd_flops * 0.2
+    elif "attn_bwd_dq" in kernels:  # both kernels recompute S and dP; credited 3 : 2 (dV, dK, + S | dQ, + dP)
         kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops * 0.6
         kernel_flops["attn_bwd_dq"] = 2.5 * fwd_flops * 0.4
     else:
@@ -240,7 +244,7 @@ def main() -> int:
     if not args.skip_extra:
         extra = {}
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
-        extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(5, args.warmup))
+        extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup))
         result["extra"] = extra
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)

@@ -204,6 +204,8 @@ extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const i
   }
   bp.accumulate_f32 = accumulate_f32 ? 1 : 0;
   bp.nkt = 0;
+  bp.ds_ws = nullptr;
+  bp.ds_nkb = bp.ds_nqt = 0;
   if (s->Sq > 0) {
     int rc = mlts_attn_delta(dout, do_stride, o, s->o_stride, delta, s->B, s->Hq, s->Sq, s->D, s->dtype, st);
     if (rc != MLTS_OK) return rc;

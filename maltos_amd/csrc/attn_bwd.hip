@@ -397,6 +397,8 @@ int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq);  
 
 int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);  // attn_bwd_split.hip
 int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
+int64_t mlts_attn_bwd_ds_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t Sk);                              // attn_bwd_dq_ds.hip
+int mlts_attn_bwd_dq_bf16_ds(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_ds.hip
 
 namespace {
 // Two-role dK/dV kernel and transpose-read dQ kernel by default; tuning aid MLTS_BWD_VARIANT=staged selects the
@@ -410,9 +412,24 @@ bool use_staged_bwd() {
 }
 }  // namespace
 
+// The dK/dV kernel can hand -dS (bf16, 2 bytes per (query, key) pair of the score matrix) over to a dQ kernel that
+// then does one matrix product instead of recomputing the scores (three).  Used without a document mask when the
+// hand-over fits the budget: MLTS_BWD_DS_MAX_MB megabytes (default 4096; 0 turns it off).
+static int64_t ds_handover_bytes(int B, int Hq, int Sq, int Sk, int D, int mode, int accumulate_f32) {
+  static const int64_t max_bytes = [] {
+    const char* e = getenv("MLTS_BWD_DS_MAX_MB");
+    return (e ? static_cast<int64_t>(atoll(e)) : int64_t{4096}) << 20;
+  }();
+  // head_dim 64 has half the matrix work per pair and the same hand-over bytes: recomputing is faster there.  Block
+  // gradients that are accumulated in fp32 (ring steps) keep the recomputed, once-rounded dS.
+  if (use_staged_bwd() || mode == MLTS_MASK_DOC || D != 128 || accumulate_f32 || Sq == 0 || Sk == 0) return 0;
+  const int64_t n = mlts_attn_bwd_ds_bytes(B, Hq, Sq, Sk);
+  return n <= max_bytes ? n : 0;
+}
+
 int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32) {
-  (void)accumulate_f32;
-  return mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);  // lse2: B*Hq*Sq + 1 floats
+  // lse2 (B*Hq*Sq + 1 floats), then the -dS hand-over
+  return mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq) + ds_handover_bytes(s->B, s->Hq, s->Sq, s->Sk, s->D, s->mask_mode, accumulate_f32);
 }
 
 int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
@@ -422,6 +439,12 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
   // the newer kernels address rows of a tile with 32-bit element offsets
   const int64_t lim = int64_t{1} << 24;
   const bool staged = use_staged_bwd() || p.qs[2] >= lim || p.ks[2] >= lim || p.vs[2] >= lim || bp.dos[2] >= lim;
+  const int64_t ds_bytes = staged ? 0 : ds_handover_bytes(p.B, p.Hq, p.Sq, p.Sk, D, mode, bp.accumulate_f32);
+  if (ds_bytes > 0) {
+    bp.ds_ws = static_cast<char*>(workspace) + mlts_attn_bwd_dkdv_split_workspace(p.B, p.Hq, p.Sq);
+    bp.ds_nkb = (p.Sk + 31) / 32;
+    bp.ds_nqt = (p.Sq + 63) / 64;
+  }
   if (!staged) {
     rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, workspace, st);
   } else if (D == 128) {
@@ -434,6 +457,7 @@ int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipSt
     else rc = launch_bwd<64, MLTS_MASK_DOC>(bp, st);
   }
   if (rc != MLTS_OK) return rc;
+  if (ds_bytes > 0) return mlts_attn_bwd_dq_bf16_ds(bp, D, mode, st);
   if (!staged) return mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
   return mlts_attn_bwd_dq_bf16(bp, D, mode, st);
 }

@@ -574,6 +574,20 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       }
     }
   };
+  // hand -dS of tile x over to the dQ kernel: four fully coalesced 1 KiB stores per wavefront
+  auto role1_ds_store = [&](const Pos& x) {
+    if (MODE == MLTS_MASK_NONE && wkv0 + 32 > p.Sk && kj >= p.Sk) {  // without a mask, keys past the end hold garbage
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dsfr[f][i] = static_cast<bf16_t>(0.f);
+    }
+    const int64_t blk = ((static_cast<int64_t>(b) * p.Hq + hkv * group + x.h) * bp.ds_nkb + (wkv0 >> 5)) * bp.ds_nqt + qt_begin + x.qt;
+    unsigned char* dst = static_cast<unsigned char*>(bp.ds_ws) + blk * 4096 + lane * 16;
+#pragma unroll
+    for (int f = 0; f < 4; ++f)  // streamed: the hand-over is read once, by another kernel, and must not evict Q/dO
+      __builtin_nontemporal_store(__builtin_bit_cast(v4i32, dsfr[f]), reinterpret_cast<v4i32*>(dst + f * 1024));
+  };
   // ---- ... and, after the dp of the next tile, -dK += (-dS)^T Q (transposed reads, while role 0 does its softmax) ----
   auto role1_dk = [&](const int stage) {
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
@@ -621,6 +635,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     int stage = 0, k = 0;
     bool prev_active = false;
     int prev_stage = 0;
+    Pos prev_it = it;
     while (!at_end(it)) {
       Pos itn = it;
       step(itn);
@@ -641,8 +656,12 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         if (prev_active) role1_dk(prev_stage);
       }
       if (!at_end(itn)) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
+      // after the wait for the next tile's loads: loads and stores complete out of order with respect to each other,
+      // so a store in front of that wait would make it wait for the store's acknowledgement as well
+      if (ROLE == 1 && prev_active && bp.ds_ws) role1_ds_store(prev_it);
       prev_active = cls != TILE_SKIP;
       prev_stage = stage;
+      prev_it = it;
       it = itn;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
       ++k;
@@ -650,6 +669,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     drain_and_barrier();
     if (ROLE == 1 && prev_active) {
       role1_ds(((k - 1) & 1) * (4 * PBUF_BYTES));
+      if (bp.ds_ws) role1_ds_store(prev_it);
       role1_dk(prev_stage);
     }
     last_stage = prev_stage;
