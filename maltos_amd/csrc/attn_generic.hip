@@ -317,6 +317,46 @@ __global__ __launch_bounds__(GT) void attn_delta_kernel(const T* __restrict__ do
   if (lane == 0) delta[row] = acc;
 }
 
+// bf16, head_dim a multiple of 8, 16-byte aligned rows: D / 8 lanes share a row (one 16-byte load of dO and of O per
+// lane), four rows per lane group in flight.  The plain kernel above reads two bytes per lane and reaches 3 TB/s.
+template <int LPR>  // lanes per row, a power of two <= 32
+__global__ __launch_bounds__(256) void attn_delta_vec_kernel(const bf16_t* __restrict__ dout, int64_t ds0, int64_t ds1, int64_t ds2,
+                                                              const bf16_t* __restrict__ o, int64_t os0, int64_t os1, int64_t os2,
+                                                              float* __restrict__ delta, int H, int S, int64_t total, int D) {
+  constexpr int RPB = 256 / LPR;  // rows per block and pass
+  constexpr int UNROLL = 4;
+  const int sub = threadIdx.x % LPR;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * (RPB * UNROLL) + threadIdx.x / LPR;
+  typedef int v4i32 __attribute__((ext_vector_type(4)));
+  v4i32 a[UNROLL], c[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t row = min(row0 + u * RPB, total - 1);
+    const int s = static_cast<int>(row % S);
+    const int h = static_cast<int>((row / S) % H);
+    const int64_t b = row / (static_cast<int64_t>(S) * H);
+    a[u] = v4i32{0, 0, 0, 0};
+    c[u] = v4i32{0, 0, 0, 0};
+    if (sub * 8 < D) {
+      a[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i32*>(dout + b * ds0 + h * ds1 + static_cast<int64_t>(s) * ds2 + sub * 8));
+      c[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i32*>(o + b * os0 + h * os1 + static_cast<int64_t>(s) * os2 + sub * 8));
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // two bf16 per 32-bit word: low half = even element
+      acc += __builtin_bit_cast(float, a[u][i] << 16) * __builtin_bit_cast(float, c[u][i] << 16);
+      acc += __builtin_bit_cast(float, a[u][i] & static_cast<int>(0xffff0000u)) * __builtin_bit_cast(float, c[u][i] & static_cast<int>(0xffff0000u));
+    }
+#pragma unroll
+    for (int m = LPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+    const int64_t row = row0 + u * RPB;
+    if (sub == 0 && row < total) delta[row] = acc;
+  }
+}
+
 template <typename KERN>
 int set_lds(KERN kern, size_t bytes, const char* what) {
   if (bytes > 48 * 1024) {
@@ -394,6 +434,22 @@ int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const i
                     int S, int D, int dtype, hipStream_t st) {
   const int64_t rows = static_cast<int64_t>(B) * H * S;
   if (rows == 0) return MLTS_OK;
+  const bool vec = dtype == MLTS_BF16 && D % 8 == 0 && D <= 256 && ((dos[0] | dos[1] | dos[2] | os[0] | os[1] | os[2]) & 7) == 0 &&
+                   mlts_aligned16(dout) && mlts_aligned16(o);
+  if (vec) {
+    const int lpr = D <= 64 ? 8 : D <= 128 ? 16 : 32;
+    const int64_t rows_per_block = (256 / lpr) * 4;
+    const unsigned nb = static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block);
+    const bf16_t* dp = static_cast<const bf16_t*>(dout);
+    const bf16_t* op = static_cast<const bf16_t*>(o);
+#define MLTS_DELTA(LPR) \
+  hipLaunchKernelGGL(attn_delta_vec_kernel<LPR>, dim3(nb), dim3(256), 0, st, dp, dos[0], dos[1], dos[2], op, os[0], os[1], os[2], delta, H, S, rows, D)
+    if (lpr == 8) MLTS_DELTA(8);
+    else if (lpr == 16) MLTS_DELTA(16);
+    else MLTS_DELTA(32);
+#undef MLTS_DELTA
+    return mlts_check_launch("mlts_attn_delta");
+  }
   const int64_t blocks = (rows + (GT / 64) - 1) / (GT / 64);
   if (dtype == MLTS_BF16)
     hipLaunchKernelGGL(attn_delta_kernel<bf16_t>, dim3((unsigned)blocks), dim3(GT), 0, st, static_cast<const bf16_t*>(dout),
