@@ -674,8 +674,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     }
     last_stage = prev_stage;
   };
-  if (role == 0) tile_loop(std::integral_constant<int, 0>{});
-  else tile_loop(std::integral_constant<int, 1>{});
+  if (role == 0) {
+    __builtin_amdgcn_s_setprio(1);  // role 0 has the longer chain per tile (softmax between its two products)
+    tile_loop(std::integral_constant<int, 0>{});
+    __builtin_amdgcn_s_setprio(0);
+  } else {
+    tile_loop(std::integral_constant<int, 1>{});
+  }
 
   // ---- write dV (role 0) or dK (role 1) ----
   {

@@ -294,6 +294,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   while (j < j_end) {
     const int jn = next_tile(j + 1);
     if (!late) sync();
+    __builtin_amdgcn_s_setprio(1);  // the matrix block of this wavefront goes ahead of the other wavefront's softmax
     if (pv_pending) pv_phase();
 
     const int kv0 = j * BN;
@@ -353,6 +354,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       }
 
     }
+    __builtin_amdgcn_s_setprio(0);
     if (late && jn < j_end) sync();
     if (cls != TILE_SKIP) {
       if (cls == TILE_MASKED) {
