@@ -406,18 +406,43 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
           for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
       }
       const float m_use = m_run == -INFINITY ? 0.f : m_run;
-      float ls = 0.f;
+      if constexpr (D == 64) {
+        // probabilities in pairs: one packed conversion and one dot product with (1, 1) per pair, so the row sum is
+        // the sum of the bf16 values that enter the PV product (measured: 5 % faster at head_dim 64, 4 % slower at
+        // 128, which keeps the plain sum below)
+        float ls4[4] = {0.f, 0.f, 0.f, 0.f};
+        const bf16x2 ones = {static_cast<bf16_t>(1.0f), static_cast<bf16_t>(1.0f)};
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < 2; ++t) {
+            v4i32 w;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float pv = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + i] * p.scale_log2 - m_use);
-            ls += pv;
-            pf[kb * 2 + t][i] = static_cast<bf16_t>(pv);
+            for (int i = 0; i < 4; ++i) {
+              f32x2 pv;
+              pv[0] = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + 2 * i] * p.scale_log2 - m_use);
+              pv[1] = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + 2 * i + 1] * p.scale_log2 - m_use);
+              const bf16x2 pb = __builtin_convertvector(pv, bf16x2);
+              ls4[i] = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, ls4[i], false);
+              w[i] = __builtin_bit_cast(int, pb);
+            }
+            pf[kb * 2 + t] = __builtin_bit_cast(bf16x8, w);
           }
-      l_run += ls;
+        l_run += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
+      } else {
+        float ls = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const float pv = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + i] * p.scale_log2 - m_use);
+              ls += pv;
+              pf[kb * 2 + t][i] = static_cast<bf16_t>(pv);
+            }
+        l_run += ls;
+      }
 
     }
     pv_pending = cls != TILE_SKIP;
