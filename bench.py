@@ -102,6 +102,21 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup):
     return sec, flops, kernels, kernel_flops
 
 
+def bench_attention_recompute(args):
+    """The same attention step with MLTS_BWD_DS_MAX_MB=0: the dQ kernel recomputes S and dP instead of reading dS from
+    the dK/dV kernel (workspace O(S) instead of 2 bytes per score).  The choice is read once per process, so this
+    runs in a child process."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--skip-extra", "--skip-cpu", "--steps", str(args.steps),
+           "--warmup", str(args.warmup)]
+    proc = subprocess.run(cmd, env={**os.environ, "MLTS_BWD_DS_MAX_MB": "0"}, capture_output=True, text=True, timeout=600)
+    if proc.returncode != 0:
+        raise RuntimeError(f"recompute-backward leg failed:\n{proc.stderr[-2000:]}")
+    r = json.loads(proc.stdout.strip().splitlines()[-1])
+    return {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "kernels": r["kernels"],
+            "workspace": "lse2 + delta + tile statistics only"}
+
+
 def bench_adamw(torch, ops, _lib, dev, steps, warmup):
     n = 58_073_600  # LLaMA-50M parameters
     p = torch.randn(n, device=dev)
@@ -246,6 +261,8 @@ def main() -> int:
     }
     if not args.skip_extra:
         extra = {}
+        if "attn_bwd_dq_ds" in kernels:
+            extra["attn_recompute_backward"] = bench_attention_recompute(args)
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
         extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup))
         result["extra"] = extra
