@@ -87,6 +87,9 @@ def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad
 CASES = [
     # B, Hq, Hkv, Sq, Sk, D, mode
     (1, 1, 1, 1, 1, 64, ops.MASK_CAUSAL),
+    (1, 1, 1, 1, 1, 128, ops.MASK_CAUSAL),
+    (2, 2, 2, 33, 65, 128, ops.MASK_NONE),
+    (1, 2, 1, 257, 257, 128, ops.MASK_CAUSAL),
     (2, 4, 4, 100, 100, 64, ops.MASK_CAUSAL),
     (1, 2, 2, 256, 256, 128, ops.MASK_CAUSAL),
     (2, 3, 3, 300, 300, 64, ops.MASK_CAUSAL),
