@@ -58,72 +58,93 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const T* __restri
 // partials live in registers (hidden <= 64 * N * kMaxChunks).
 constexpr int kMaxChunks = 8;
 
-template <typename T>
+// CH = 16-byte chunks per lane and row (1, 2, 4 or 8); 8 / CH rows of a wavefront are in flight at once and their
+// vectors stay in registers between the two passes (one row at a time leaves the memory latency of every row exposed).
+template <typename T, int CH>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                                                                const T* __restrict__ w, const float* __restrict__ rstd,
                                                                T* __restrict__ dx, float* __restrict__ dw_partial,
                                                                int64_t rows, int hidden, int rows_per_block) {
   constexpr int N = Vec16<T>::N;
+  constexpr int R = 8 / CH;
   extern __shared__ float smem[];  // [kWaves][hidden]
   const int lane = threadIdx.x & (MLTS_WAVE - 1);
   const int wave = threadIdx.x / MLTS_WAVE;
   const int nvec = hidden / N;
-  const int chunks = (nvec + MLTS_WAVE - 1) / MLTS_WAVE;
-  float dwacc[kMaxChunks][N];
+  constexpr int chunks = CH;
+  float dwacc[CH][N];
+  Vec16<T> wv[CH];
 #pragma unroll
-  for (int c = 0; c < kMaxChunks; ++c)
+  for (int c = 0; c < CH; ++c) {
 #pragma unroll
     for (int j = 0; j < N; ++j) dwacc[c][j] = 0.f;
+    const int col = lane + c * MLTS_WAVE;
+    if (col < nvec) wv[c] = reinterpret_cast<const Vec16<T>*>(w)[col];
+  }
 
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rows_per_block;
   int64_t row_end = row0 + rows_per_block;
   if (row_end > rows) row_end = rows;
   const float inv_h = 1.0f / static_cast<float>(hidden);
-  for (int64_t row = row0 + wave; row < row_end; row += kWaves) {
-    const float r = rstd[row];
-    const T* xr = x + row * hidden;
-    const T* dyr = dy + row * hidden;
-    T* dxr = dx + row * hidden;
-    float dot = 0.f;
+  for (int64_t row = row0 + wave; row < row_end; row += kWaves * R) {
+    Vec16<T> xv[R][CH], dv[R][CH];
+    float rr[R];
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-      const int col = lane + c * MLTS_WAVE;
-      if (c < chunks && col < nvec) {
-        Vec16<T> xv = reinterpret_cast<const Vec16<T>*>(xr)[col];
-        Vec16<T> dv = reinterpret_cast<const Vec16<T>*>(dyr)[col];
-        Vec16<T> wv = reinterpret_cast<const Vec16<T>*>(w)[col];
+    for (int i = 0; i < R; ++i) {
+      int64_t ri = row + static_cast<int64_t>(i) * kWaves;
+      if (ri >= row_end) ri = row;  // loaded again, not used
+      rr[i] = rstd[ri];
 #pragma unroll
-        for (int j = 0; j < N; ++j) {
-          float xh = xv.get(j) * r;
-          float d = dv.get(j);
-          dwacc[c][j] += d * xh;
-          dot += d * wv.get(j) * xh;
+      for (int c = 0; c < CH; ++c) {
+        const int col = lane + c * MLTS_WAVE;
+        if (col < nvec) {
+          xv[i][c] = reinterpret_cast<const Vec16<T>*>(x + ri * hidden)[col];
+          dv[i][c] = reinterpret_cast<const Vec16<T>*>(dy + ri * hidden)[col];
         }
       }
     }
-    dot = wave_sum(dot) * inv_h;
 #pragma unroll
-    for (int c = 0; c < kMaxChunks; ++c) {
-      const int col = lane + c * MLTS_WAVE;
-      if (c < chunks && col < nvec) {
-        Vec16<T> xv = reinterpret_cast<const Vec16<T>*>(xr)[col];
-        Vec16<T> dv = reinterpret_cast<const Vec16<T>*>(dyr)[col];
-        Vec16<T> wv = reinterpret_cast<const Vec16<T>*>(w)[col];
-        Vec16<T> o;
+    for (int i = 0; i < R; ++i) {
+      const int64_t ri = row + static_cast<int64_t>(i) * kWaves;
+      if (ri < row_end) {
+        const float r = rr[i];
+        float dot = 0.f;
 #pragma unroll
-        for (int j = 0; j < N; ++j) {
-          float xh = xv.get(j) * r;
-          o.set(j, r * (dv.get(j) * wv.get(j) - xh * dot));
+        for (int c = 0; c < CH; ++c) {
+          const int col = lane + c * MLTS_WAVE;
+          if (col < nvec) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+              float xh = xv[i][c].get(j) * r;
+              float d = dv[i][c].get(j);
+              dwacc[c][j] += d * xh;
+              dot += d * wv[c].get(j) * xh;
+            }
+          }
         }
-        reinterpret_cast<Vec16<T>*>(dxr)[col] = o;
+        dot = wave_sum(dot) * inv_h;
+        T* dxr = dx + ri * hidden;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+          const int col = lane + c * MLTS_WAVE;
+          if (col < nvec) {
+            Vec16<T> o;
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+              float xh = xv[i][c].get(j) * r;
+              o.set(j, r * (dv[i][c].get(j) * wv[c].get(j) - xh * dot));
+            }
+            reinterpret_cast<Vec16<T>*>(dxr)[col] = o;
+          }
+        }
       }
     }
   }
   // reduce the four waves' dw partials through LDS
 #pragma unroll
-  for (int c = 0; c < kMaxChunks; ++c) {
+  for (int c = 0; c < chunks; ++c) {
     const int col = lane + c * MLTS_WAVE;
-    if (c < chunks && col < nvec) {
+    if (col < nvec) {
 #pragma unroll
       for (int j = 0; j < N; ++j) smem[wave * hidden + col * N + j] = dwacc[c][j];
     }
@@ -132,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restri
   for (int i = threadIdx.x; i < hidden; i += kThreads) {
     float s = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < kWaves; ++wv) s += smem[wv * hidden + i];
+    for (int wi = 0; wi < kWaves; ++wi) s += smem[wi * hidden + i];
     dw_partial[static_cast<int64_t>(blockIdx.x) * hidden + i] = s;
   }
 }
@@ -168,7 +189,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_dw_reduce_kernel(const float
 
 int rmsnorm_bwd_blocks(int64_t rows) {
   int64_t b = (rows + 31) / 32;  // >= 32 rows per block keeps the partial buffer small
-  if (b > 256) b = 256;          // one block per CU; more only lengthens the reduction above
+  if (b > 256) b = 256;          // one block per CU; more (tried: 1024) only lengthens the reduction above
   if (b < 1) b = 1;
   return static_cast<int>(b);
 }
@@ -309,9 +330,16 @@ int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rst
   const int rows_per_block = static_cast<int>((rows + blocks - 1) / blocks);
   const size_t smem = static_cast<size_t>(kWaves) * hidden * sizeof(float);
   MltsKernelTimer timer("rmsnorm_bwd", st);
-  hipLaunchKernelGGL(rmsnorm_bwd_kernel<T>, dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy),
-                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,
-                     hidden, rows_per_block);
+  const int chunks = (hidden / Vec16<T>::N + MLTS_WAVE - 1) / MLTS_WAVE;  // <= kMaxChunks, checked by the caller
+#define MLTS_RMS_BWD(CH)                                                                                              \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH>), dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy), \
+                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,   \
+                     hidden, rows_per_block)
+  if (chunks <= 1) MLTS_RMS_BWD(1);
+  else if (chunks <= 2) MLTS_RMS_BWD(2);
+  else if (chunks <= 4) MLTS_RMS_BWD(4);
+  else MLTS_RMS_BWD(8);
+#undef MLTS_RMS_BWD
   hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + 31) / 32), dim3(kThreads), 0, st,
                      partial, blocks, hidden, static_cast<T*>(dw));
   return mlts_check_launch("mlts_rmsnorm_bwd");
