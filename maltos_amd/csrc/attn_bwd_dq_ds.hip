@@ -1,4 +1,4 @@
-// Attention backward, dQ from the -dS blocks that the dK/dV kernel hands over, head_dim 64 and 128, bf16.
+// Attention backward, dQ from the -dS blocks that the dK/dV kernel hands over, head_dim 128, bf16.
 //
 // The two-kernel backward computes the scores twice (once per kernel).  When the caller's workspace has room for
 // -dS (bf16, one value per visible (query, key) pair), the dK/dV kernel stores it and this kernel only does
@@ -338,8 +338,12 @@ int64_t mlts_attn_bwd_ds_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t Sk) {
   return B * Hq * ((Sk + 31) / 32) * ((Sq + 63) / 64) * 4096;
 }
 
-// head_dim 64 or 128, MLTS_MASK_NONE or MLTS_MASK_CAUSAL, bp.ds_ws filled by the dK/dV kernel on the same stream
+// head_dim 128 (at 64 the recomputing kernel is faster and the caller never hands dS over), MLTS_MASK_NONE or
+// MLTS_MASK_CAUSAL, bp.ds_ws filled by the dK/dV kernel on the same stream
 int mlts_attn_bwd_dq_bf16_ds(const AttnBwdParams& bp, int D, int mode, hipStream_t st) {
-  if (mode == MLTS_MASK_CAUSAL) return D == 128 ? launch<128, true>(bp, st) : launch<64, true>(bp, st);
-  return D == 128 ? launch<128, false>(bp, st) : launch<64, false>(bp, st);
+  if (D != 128 || mode == MLTS_MASK_DOC || !bp.ds_ws) {
+    mlts_set_error("mlts_attn_bwd: the dS hand-over kernel needs head_dim 128, no document mask and a hand-over buffer");
+    return MLTS_ERR_UNSUPPORTED;
+  }
+  return mode == MLTS_MASK_CAUSAL ? launch<128, true>(bp, st) : launch<128, false>(bp, st);
 }
