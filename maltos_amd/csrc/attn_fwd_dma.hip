@@ -86,6 +86,12 @@ __device__ __forceinline__ bf16x8 as_frag(v2i32 lo, v2i32 hi) {
   return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
 }
 
+// x of this lane and of lane ^ 32, without the LDS round trip of a bpermute: v_permlane32_swap exchanges the upper
+// half of one register with the lower half of another
+__device__ __forceinline__ void both_halves(float x, float& lo, float& hi) {
+  asm("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %2\n\ts_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "=&v"(lo), "=&v"(hi) : "v"(x));
+}
+
 template <int D, int MODE>
 __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams p) {
   using C = FwdCfg<D>;
@@ -392,7 +398,11 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * p.scale_log2;
+      {
+        float mlo, mhi;
+        both_halves(mx, mlo, mhi);
+        mx = fmaxf(mlo, mhi) * p.scale_log2;
+      }
       const bool raise = mx > m_run + 8.0f;  // also true for the first visible tile (m_run = -inf)
       if (__builtin_amdgcn_ballot_w64(raise) != 0) {
         const float m_new = raise ? mx : m_run;
@@ -452,7 +462,9 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   }
   if (pv_pending) pv_phase();
 
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  float l_lo, l_hi;
+  both_halves(l_run, l_lo, l_hi);
+  const float l_tot = l_lo + l_hi;
   const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
   if (qrow < p.Sq && hh == 0) {
     p.lse[(static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow] =
