@@ -146,7 +146,9 @@ def bench_adamw(torch, ops, _lib, dev, steps, warmup):
             "frac_of_hbm_peak": bytes_per_launch / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
-def bench_llama50m(torch, dev, steps, warmup):
+def bench_llama50m(torch, dev, steps, warmup, zero1=False):
+    """zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
+    per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer."""
     from maltos_amd.grad_clip import clip_grad_norm_fused_
     from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
     from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
@@ -160,8 +162,13 @@ def bench_llama50m(torch, dev, steps, warmup):
             if p.dim() >= 2:
                 p.normal_(0.0, 0.02)
     model = model.to(dev).to(torch.bfloat16)
-    opt = MasterWeightsOptimizer(model.parameters(), optimizer_factory=lambda ps: FusedAdamW(
+    factory = lambda params: MasterWeightsOptimizer(params, optimizer_factory=lambda ps: FusedAdamW(
         ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1))
+    if zero1:
+        from maltos_amd.zero1 import Zero1FlatBuffers
+        z = Zero1FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=25)
+    else:
+        opt = factory(model.parameters())
     gen = torch.Generator().manual_seed(1234)
     ids = torch.randint(0, cfg.vocab_size, (8, 2049), generator=gen).to(dev)
     batch = {"input_ids": ids[:, :-1].contiguous(), "labels": ids[:, 1:].contiguous()}
@@ -175,11 +182,22 @@ def bench_llama50m(torch, dev, steps, warmup):
         opt.zero_grad(set_to_none=True)
         out["loss"] = loss
 
-    sec = timed(torch, step, steps, warmup)
+    def step_zero1():
+        z.reset_grads()
+        loss = model(batch)
+        loss.backward()
+        out["norm"] = z.step(1.0)
+        out["loss"] = loss
+
+    sec = timed(torch, step_zero1 if zero1 else step, steps, warmup)
     tokens = 8 * 2048
-    return {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"]),
-            "grad_norm_last": float(out["sq"].sqrt()), "params": sum(p.numel() for p in model.parameters()),
-            "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12}
+    res = {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"].detach()),
+           "grad_norm_last": float(out["norm"]) if zero1 else float(out["sq"].sqrt()),
+           "params": sum(p.numel() for p in model.parameters()),
+           "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12}
+    if zero1:
+        res["buckets"] = len(z.buckets)
+    return res
 
 
 def cpu_baseline(torch):
@@ -265,6 +283,8 @@ def main() -> int:
             extra["attn_recompute_backward"] = bench_attention_recompute(args)
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
         extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup))
+        extra["llama50m_train_step_zero1_layout"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup),
+                                                                   zero1=True)
         result["extra"] = extra
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)

@@ -146,3 +146,33 @@ def test_non_finite_norm_raises(dev):
     next(model.parameters()).grad[0, 0] = float("inf")
     with pytest.raises(FloatingPointError):
         clip_grad_norm_(opt, 1.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_zero1_flat_buffers_step_equals_plain_optimizer(dev, dtype):
+    """The fused optimizer inside the ZeRO-1 layout (reverse-order buckets, flat data/grad buffers, per-bucket local
+    shards; world_size 1) takes the same steps as the same optimizer on the model's own parameters: AdamW is
+    elementwise, so only the clip coefficient (an fp64 sum in another order) can differ, in its last bits."""
+    from maltos_amd.zero1 import Zero1FlatBuffers
+
+    plain_model = _model(dev, dtype)
+    zero_model = copy.deepcopy(plain_model)
+    inner = lambda ps: FusedAdamW(ps, **HP)
+    factory = (lambda ps: MasterWeightsOptimizer(ps, optimizer_factory=inner)) if dtype == torch.bfloat16 else inner
+    plain = factory(list(plain_model.parameters()))
+    z = Zero1FlatBuffers(zero_model, optimizer_factory=factory, bucket_mb_size=25)
+    assert sum(len(b.params) for b in z.buckets) == len(list(zero_model.parameters()))
+    max_norm = 0.5
+    for step in range(3):
+        x = torch.randn(16, 24, device=dev, dtype=dtype, generator=torch.Generator(device=dev).manual_seed(step))
+        _loss(plain_model, x).backward()
+        want_norm = clip_grad_norm_(plain, max_norm)
+        plain.step()
+        plain.zero_grad(set_to_none=True)
+        z.reset_grads()
+        _loss(zero_model, x).backward()
+        got_norm = z.step(max_norm)
+        assert got_norm == pytest.approx(want_norm, rel=1e-6)
+        for p, q in zip(zero_model.parameters(), plain_model.parameters()):
+            assert p.data_ptr() >= z.data_buffer.data_ptr()  # still a view of the flat buffer
+            torch.testing.assert_close(p.detach().float(), q.detach().float(), rtol=1e-5 if dtype == torch.float32 else 2 ** -7, atol=1e-7)
