@@ -409,3 +409,43 @@ def test_kernel_variants_agree(dev, tmp_path):
             for what, a, b in zip(("O", "LSE", "dQ", "dK", "dV"), results[tag][name], want):
                 assert torch.isfinite(a).all()
                 assert ((a - b).abs() <= 2e-2 + 2.0 ** -7 * b.abs()).all(), f"{tag} {name} {what}: {(a - b).abs().max().item():.3e}"
+
+
+@pytest.mark.parametrize("packed", [False, True], ids=["positions-only", "packed-documents"])
+def test_all_gather_kv_core_matches_global_attention(dev, packed):
+    """Every rank's local queries over the gathered keys equal global (document-)causal attention at the rank's tokens,
+    forward and backward; chunks are the zigzag split, so the gathered keys are not in position order."""
+    from maltos_amd.all_gather_attention import HipAllGatherKvAttentionCore
+
+    world_size, s_loc, B, Hq, Hkv, D = 4, 128, 2, 4, 2, 128
+    total = world_size * s_loc
+    gen = torch.Generator().manual_seed(77 + packed)
+    all_q, all_k, all_v = bshd(B, Hq, total, D, gen, torch.bfloat16), bshd(B, Hkv, total, D, gen, torch.bfloat16), bshd(B, Hkv, total, D, gen, torch.bfloat16)
+    if packed:
+        all_pos, all_seq = make_docs(B, total, gen, 200, pad_tail=19)
+        mask = oa.doc_mask(all_pos, all_pos, all_seq, all_seq)
+    else:
+        all_pos, all_seq = torch.arange(total).expand(B, total).contiguous(), None
+        mask = oa.causal_mask(total, total, "cpu")
+    idx = [expected_zigzag_ring_positions(s_loc, rank=r, world_size=world_size, device=torch.device("cpu")) for r in range(world_size)]
+    gq, gk, gv = (t.detach().float().clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, _ = oa.attention_with_lse(gq, gk, gv, mask)
+    dout_all = torch.randn(gout.shape, generator=gen).bfloat16()
+    gout.backward(dout_all.float())
+    dk_sum, dv_sum = torch.zeros_like(gk.grad), torch.zeros_like(gv.grad)
+    pc = [all_pos.index_select(1, i).to(dev) for i in idx]
+    sc = [all_seq.index_select(1, i).to(dev) if packed else None for i in idx]
+    for rank in range(world_size):
+        q = all_q.index_select(2, idx[rank]).to(dev).requires_grad_(True)
+        chunks = [(all_k.index_select(2, i).to(dev).requires_grad_(True), all_v.index_select(2, i).to(dev).requires_grad_(True)) for i in idx]
+        core = HipAllGatherKvAttentionCore(rank=rank, world_size=world_size, kv_source=lambda r, k, v, c=chunks: c,
+                                           meta_source=lambda r, p, s: list(zip(pc, sc)))
+        out = core(q, chunks[rank][0], chunks[rank][1], 0, pc[rank], sc[rank])
+        check(out, gout.detach().index_select(2, idx[rank]), torch.bfloat16, f"all-gather O rank{rank}")
+        out.backward(dout_all.index_select(2, idx[rank]).to(dev))
+        check(q.grad, gq.grad.index_select(2, idx[rank]), torch.bfloat16, f"all-gather dQ rank{rank}")
+        for src, (k, v) in enumerate(chunks):
+            dk_sum.index_add_(2, idx[src], k.grad.float().cpu())
+            dv_sum.index_add_(2, idx[src], v.grad.float().cpu())
+    assert ((dk_sum - gk.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gk.grad.abs())).all()
+    assert ((dv_sum - gv.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gv.grad.abs())).all()
