@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled
 # by the same counters over the --calibrate-traffic kernel (summary: profiles/attn_cfg2_hbm_traffic.md).  Counters
 # cannot be read from inside the timed run, so the figures are carried here and refreshed with the profile.
-MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 628.9e6, "attn_bwd_dkdv": 1967.6e6, "attn_bwd_dq_ds": 1426.2e6,
+MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 679.1e6, "attn_bwd_dkdv": 1965.8e6, "attn_bwd_dq_ds": 1425.9e6,
                               # the recomputing dQ kernel and the dK/dV kernel without the dS hand-over (MLTS_BWD_DS_MAX_MB=0)
                               "attn_bwd_dq": 651.3e6, "attn_bwd_dkdv_recompute": 885.8e6}
 
