@@ -50,14 +50,22 @@ def attention_inputs(torch, dev, B, H, S, D, seed=1234):
 
 
 def timed(torch, fn, steps, warmup):
+    """Mean seconds per call.  The interpreter's cyclic garbage collector is held off during the timed calls (as
+    timeit does): one full collection is a 50-100 ms pause, which in a launch-bound loop of ten steps is the result."""
+    import gc
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
+    gc.collect()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+    finally:
+        gc.enable()
 
 
 def bench_attention(torch, ops, _lib, dev, steps, warmup):
@@ -146,11 +154,12 @@ def bench_adamw(torch, ops, _lib, dev, steps, warmup):
             "frac_of_hbm_peak": bytes_per_launch / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
-def bench_llama50m(torch, dev, steps, warmup, zero1=False):
-    """zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
+def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False):
+    """graph=True: forward + backward replayed from one HIP graph (clip, AdamW and the gradient clear stay eager).
+    zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
     per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer."""
     from maltos_amd.grad_clip import clip_grad_norm_fused_
-    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
     from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
 
     cfg = LlamaConfig(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8,
@@ -162,6 +171,7 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False):
             if p.dim() >= 2:
                 p.normal_(0.0, 0.02)
     model = model.to(dev).to(torch.bfloat16)
+    set_grad_accumulation_into_buffers(model)  # gradients live in flat buffers that are cleared in place: dW adds into them
     factory = lambda params: MasterWeightsOptimizer(params, optimizer_factory=lambda ps: FusedAdamW(
         ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1))
     if zero1:
@@ -182,6 +192,16 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False):
         opt.zero_grad(set_to_none=True)
         out["loss"] = loss
 
+    if graph:
+        from maltos_amd.graph_step import CapturedForwardBackward
+        captured = CapturedForwardBackward(model, batch, embed=model.embed_tokens, clear_grads=lambda: opt.zero_grad(set_to_none=True))
+
+    def step_graph():
+        out["loss"] = captured(batch)
+        out["sq"] = clip_grad_norm_fused_(opt, 1.0)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+
     def step_zero1():
         z.reset_grads()
         loss = model(batch)
@@ -189,7 +209,7 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False):
         out["norm"] = z.step(1.0)
         out["loss"] = loss
 
-    sec = timed(torch, step_zero1 if zero1 else step, steps, warmup)
+    sec = timed(torch, step_zero1 if zero1 else step_graph if graph else step, steps, warmup)
     tokens = 8 * 2048
     res = {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"].detach()),
            "grad_norm_last": float(out["norm"]) if zero1 else float(out["sq"].sqrt()),
@@ -283,6 +303,7 @@ def main() -> int:
             extra["attn_recompute_backward"] = bench_attention_recompute(args)
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
         extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup))
+        extra["llama50m_train_step_graph"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup), graph=True)
         extra["llama50m_train_step_zero1_layout"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup),
                                                                    zero1=True)
         result["extra"] = extra

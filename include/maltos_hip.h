@@ -170,6 +170,14 @@ int mlts_scale_by_device_scalar(void* x, const float* scale, int64_t n, int32_t 
 int mlts_grad_to_f32(float* dst, const void* src, int32_t src_dtype, int64_t n, int accumulate, double* sq_out,
                      void* workspace, mlts_stream_t stream);
 
+/* out[i] = (accumulate ? out[i] : 0) + sum over s < slices of parts[s * n + i], added in fp32 and rounded once to
+ * `dtype` (bf16 or fp32; out and parts share it).  Finishes a weight gradient dW = dY^T X of nn.Linear
+ * (models/llama.py:69-75,196-198) that was computed as `slices` row-slice products, and with accumulate != 0 adds it
+ * onto the gradient already held in a view of the flat gradient buffer (runtime/plugins/zero1.py:117-121), which is
+ * what autograd's `param.grad += dW` does there in a second pass. */
+int mlts_grad_sum_slices(void* out, const void* parts, int32_t dtype, int32_t slices, int64_t n, int accumulate,
+                         mlts_stream_t stream);
+
 /* *sq_out = sum x[i]^2 accumulated in fp64 (runtime/plugins/grad_clip.py:62-77,
  * runtime/plugins/zero_common.py:324-329).  workspace: MLTS_SQNORM_WS_BYTES. */
 int mlts_sq_norm(const float* x, int64_t n, double* sq_out, void* workspace, mlts_stream_t stream);

@@ -90,6 +90,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_ce_fwd_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int32, C.c_int64, C.c_int32, _P]),
     "mlts_scale_by_device_scalar": (C.c_int, [_P, _P, C.c_int64, C.c_int32, _P]),
     "mlts_grad_to_f32": (C.c_int, [_P, _P, C.c_int32, C.c_int64, C.c_int, _P, _P, _P]),
+    "mlts_grad_sum_slices": (C.c_int, [_P, _P, C.c_int32, C.c_int32, C.c_int64, C.c_int, _P]),
     "mlts_sq_norm": (C.c_int, [_P, C.c_int64, _P, _P, _P]),
     "mlts_scale": (C.c_int, [_P, C.c_float, C.c_int64, _P]),
     "mlts_adamw_step": (

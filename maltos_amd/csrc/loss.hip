@@ -170,6 +170,24 @@ __global__ __launch_bounds__(256) void scale_by_scalar_kernel(T* x, const float*
     x[i] = from_f32<T>(to_f32<T>(x[i]) * s);
 }
 
+// 16-byte form for an aligned buffer: n_vec whole vectors, the tail (< one vector) by the first lanes of block 0.
+template <typename T>
+__global__ __launch_bounds__(256) void scale_by_scalar_vec_kernel(T* x, const float* scale, int64_t n_vec, int64_t n) {
+  using V = Vec16<T>;
+  const float s = *scale;
+  if (s == 1.0f) return;
+  V* xv = reinterpret_cast<V*>(x);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n_vec; i += stride) {
+    V v = xv[i];
+#pragma unroll
+    for (int j = 0; j < V::N; ++j) v.set(j, v.get(j) * s);
+    xv[i] = v;
+  }
+  const int64_t tail = n_vec * V::N + static_cast<int64_t>(threadIdx.x);
+  if (blockIdx.x == 0 && tail < n) x[tail] = from_f32<T>(to_f32<T>(x[tail]) * s);
+}
+
 constexpr int64_t kMaxStagedBytes = 128 * 1024;
 
 template <typename T>
@@ -238,6 +256,17 @@ extern "C" int mlts_scale_by_device_scalar(void* x, const float* scale, int64_t 
   if (n == 0) return MLTS_OK;
   MLTS_REQUIRE(x && scale, "mlts_scale_by_device_scalar: null pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (mlts_aligned16(x)) {
+    const int64_t per = dtype == MLTS_BF16 ? 8 : 4;
+    const int64_t n_vec = n / per;
+    int64_t blocks = (n_vec + 255) / 256;
+    blocks = blocks < 1 ? 1 : (blocks > 8192 ? 8192 : blocks);
+    if (dtype == MLTS_BF16)
+      hipLaunchKernelGGL(scale_by_scalar_vec_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, static_cast<bf16_t*>(x), scale, n_vec, n);
+    else
+      hipLaunchKernelGGL(scale_by_scalar_vec_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, static_cast<float*>(x), scale, n_vec, n);
+    return mlts_check_launch("mlts_scale_by_device_scalar");
+  }
   int64_t blocks = (n + 255) / 256;
   if (blocks > 16384) blocks = 16384;
   if (dtype == MLTS_BF16)

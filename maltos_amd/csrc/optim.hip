@@ -320,7 +320,83 @@ void launch_grad_bf16_vec(bool acc, bool sq, int blocks, hipStream_t st, float* 
   else
     hipLaunchKernelGGL((grad_bf16_to_f32_vec_kernel<false, false>), dim3(blocks), dim3(kThreads), 0, st, dst, src, nvec8, partial);
 }
+// out[i] = T((ACC ? float(out[i]) : 0) + sum_s float(parts[s * n + i])): the row-slice partial products of a weight
+// gradient added in fp32 and rounded once, optionally onto the gradient already in the buffer.
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kThreads) void grad_sum_slices_vec_kernel(T* __restrict__ out, const T* __restrict__ parts, int slices,
+                                                                       int64_t nvec) {
+  using V = Vec16<T>;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  const V* pv = reinterpret_cast<const V*>(parts);
+  V* ov = reinterpret_cast<V*>(out);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < nvec; i += stride) {
+    float acc[V::N];
+    if (ACC) {
+      const V o = ov[i];
+#pragma unroll
+      for (int j = 0; j < V::N; ++j) acc[j] = o.get(j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < V::N; ++j) acc[j] = 0.f;
+    }
+    for (int s = 0; s < slices; ++s) {
+      const V p = pv[static_cast<int64_t>(s) * nvec + i];
+#pragma unroll
+      for (int j = 0; j < V::N; ++j) acc[j] += p.get(j);
+    }
+    V r;
+#pragma unroll
+    for (int j = 0; j < V::N; ++j) r.set(j, acc[j]);
+    ov[i] = r;
+  }
+}
+
+template <typename T, bool ACC>
+__global__ __launch_bounds__(kThreads) void grad_sum_slices_kernel(T* __restrict__ out, const T* __restrict__ parts, int slices, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+    float acc = ACC ? to_f32<T>(out[i]) : 0.f;
+    for (int s = 0; s < slices; ++s) acc += to_f32<T>(parts[static_cast<int64_t>(s) * n + i]);
+    out[i] = from_f32<T>(acc);
+  }
+}
+
+template <typename T>
+void launch_grad_sum_slices(void* out, const void* parts, int slices, int64_t n, bool acc, hipStream_t st) {
+  constexpr int N = Vec16<T>::N;
+  T* o = static_cast<T*>(out);
+  const T* p = static_cast<const T*>(parts);
+  if (n % N == 0 && mlts_aligned16(out) && mlts_aligned16(parts)) {
+    const int64_t nvec = n / N;
+    const int blocks = grid_for(nvec, 4096);
+    if (acc)
+      hipLaunchKernelGGL((grad_sum_slices_vec_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, st, o, p, slices, nvec);
+    else
+      hipLaunchKernelGGL((grad_sum_slices_vec_kernel<T, false>), dim3(blocks), dim3(kThreads), 0, st, o, p, slices, nvec);
+  } else {
+    const int blocks = grid_for(n, 4096);
+    if (acc)
+      hipLaunchKernelGGL((grad_sum_slices_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, st, o, p, slices, n);
+    else
+      hipLaunchKernelGGL((grad_sum_slices_kernel<T, false>), dim3(blocks), dim3(kThreads), 0, st, o, p, slices, n);
+  }
+}
 }  // namespace
+
+extern "C" int mlts_grad_sum_slices(void* out, const void* parts, int32_t dtype, int32_t slices, int64_t n, int accumulate,
+                                   mlts_stream_t stream) {
+  MLTS_REQUIRE(dtype == MLTS_F32 || dtype == MLTS_BF16, "mlts_grad_sum_slices: unknown dtype %d", dtype);
+  MLTS_REQUIRE(n >= 0 && slices >= 1, "mlts_grad_sum_slices: n must be >= 0 and slices >= 1");
+  if (n == 0) return MLTS_OK;
+  MLTS_REQUIRE(out && parts, "mlts_grad_sum_slices: out and parts must be non-null");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MltsKernelTimer timer("grad_sum_slices", st);
+  if (dtype == MLTS_BF16)
+    launch_grad_sum_slices<bf16_t>(out, parts, slices, n, accumulate != 0, st);
+  else
+    launch_grad_sum_slices<float>(out, parts, slices, n, accumulate != 0, st);
+  return mlts_check_launch("mlts_grad_sum_slices");
+}
 
 extern "C" int mlts_grad_to_f32(float* dst, const void* src, int32_t src_dtype, int64_t n, int accumulate,
                                 double* sq_out, void* workspace, mlts_stream_t stream) {

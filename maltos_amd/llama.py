@@ -54,8 +54,9 @@ def _weight_grad_splits(rows: int, out_features: int, in_features: int) -> int:
 
 class _SplitKLinearFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    def forward(ctx, x: torch.Tensor, weight: torch.Tensor, into_grad: bool) -> torch.Tensor:
         ctx.save_for_backward(x, weight)
+        ctx.into_grad = into_grad
         return F.linear(x, weight)
 
     @staticmethod
@@ -67,24 +68,51 @@ class _SplitKLinearFn(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             x2 = x.reshape(-1, x.shape[-1])
             dy2 = dy.reshape(-1, dy.shape[-1])
+            # the gradient buffer this weight already owns (a view of a flat gradient buffer): add into it here, in
+            # the pass that finishes dW, instead of handing dW to autograd for a separate `grad += dW`
+            grad = weight.grad if ctx.into_grad else None
+            if grad is not None and not (grad.is_contiguous() and grad.dtype == weight.dtype and grad.shape == weight.shape):
+                grad = None
             splits = _weight_grad_splits(x2.shape[0], dy2.shape[1], x2.shape[1])
             if splits > 1 and x2.is_contiguous() and dy2.is_contiguous():
                 rows = x2.shape[0] // splits
                 part = torch.bmm(dy2.view(splits, rows, -1).transpose(1, 2), x2.view(splits, rows, -1))
-                dw = part.sum(0, dtype=torch.float32).to(weight.dtype)  # slices added in fp32, rounded once
+                if grad is not None:
+                    ops.grad_sum_slices(part, grad, accumulate=True)    # fp32 sum of slices + old grad, rounded once
+                else:
+                    dw = ops.grad_sum_slices(part)                      # slices added in fp32, rounded once
+            elif grad is not None:
+                grad.addmm_(dy2.t(), x2)
             else:
                 dw = dy2.t().matmul(x2)
-        return dx, dw
+        return dx, dw, None
 
 
 class HipLinear(nn.Linear):
     """nn.Linear (same parameter name and init) whose weight gradient is computed as a batch of row slices when the
-    output is too small to fill the chip (reference: plain nn.Linear, models/llama.py:69-75,196-198)."""
+    output is too small to fill the chip (reference: plain nn.Linear, models/llama.py:69-75,196-198).
+
+    `accumulate_into_grad = True` (off by default; set it on the class or on an instance) makes the backward add dW
+    straight into an existing `weight.grad` and return no gradient for the weight: one pass instead of two when the
+    gradients live in a flat buffer that is cleared, not dropped, between steps.  Autograd hooks on the weight do not
+    fire in that mode, so it is for callers that read the gradients from the buffer after backward."""
+
+    accumulate_into_grad = False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.bias is not None or not x.is_cuda:
             return F.linear(x, self.weight, self.bias)
-        return _SplitKLinearFn.apply(x, self.weight)
+        return _SplitKLinearFn.apply(x, self.weight, bool(self.accumulate_into_grad))
+
+
+def set_grad_accumulation_into_buffers(model: nn.Module, enabled: bool = True) -> int:
+    """Switches `HipLinear.accumulate_into_grad` on every HipLinear of `model`; returns how many were switched."""
+    count = 0
+    for module in model.modules():
+        if isinstance(module, HipLinear):
+            module.accumulate_into_grad = bool(enabled)
+            count += 1
+    return count
 
 
 class LlamaRMSNorm(nn.Module):

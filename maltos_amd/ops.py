@@ -304,6 +304,7 @@ _LIBRARY.define("swiglu_fwd(Tensor gate, Tensor up) -> Tensor")
 _LIBRARY.define("swiglu_bwd(Tensor dh, Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _LIBRARY.define("ce_fwd_bwd(Tensor logits, Tensor labels, int ignore_index) -> (Tensor, Tensor, Tensor)")
 _LIBRARY.define("scale_by_scalar(Tensor x, Tensor scale) -> Tensor")
+_LIBRARY.define("scale_by_scalar_(Tensor(a!) x, Tensor scale) -> ()")
 
 
 def _impl(name: str):
@@ -322,7 +323,7 @@ def _cpu_refusal(name: str) -> None:
 
 
 for _name in ("attn_fwd", "attn_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "ce_fwd_bwd",
-              "scale_by_scalar"):
+              "scale_by_scalar", "scale_by_scalar_"):
     _cpu_refusal(_name)
 
 
@@ -352,6 +353,15 @@ def _scale_by_scalar_op(x, scale):
     s = scale.to(torch.float32).reshape(1)
     _lib.check(_lib.lib().mlts_scale_by_device_scalar(_p(out), _p(s), out.numel(), _dtype_code(out), _stream()))
     return out
+
+
+@_impl("scale_by_scalar_")
+def _scale_by_scalar_inplace_op(x, scale):
+    _require_gpu(x, scale)
+    if not x.is_contiguous():
+        raise ValueError("scale_by_scalar_ needs a contiguous tensor")
+    s = scale.to(torch.float32).reshape(1)
+    _lib.check(_lib.lib().mlts_scale_by_device_scalar(_p(x), _p(s), x.numel(), _dtype_code(x), _stream()))
 
 
 # fake (meta) kernels: shapes/dtypes only, so the ops can be traced or captured
@@ -404,6 +414,11 @@ def _(logits, labels, ignore_index):
 @torch.library.register_fake("maltos::scale_by_scalar")
 def _(x, scale):
     return torch.empty_like(x)
+
+
+@torch.library.register_fake("maltos::scale_by_scalar_")
+def _(x, scale):
+    return None
 
 
 # --------------------------------------------------------------------------------------------
@@ -468,11 +483,22 @@ torch.library.register_autograd("maltos::swiglu_fwd", _swiglu_backward, setup_co
 
 def _ce_setup(ctx, inputs, output):
     ctx.save_for_backward(output[1])
+    ctx.set_materialize_grads(False)   # no zero tensor of the logits' size for the unused dlogits output
+    ctx.dlogits_consumed = False
 
 
 def _ce_backward(ctx, dloss, _ddlogits, _dcount):
+    """d loss / d logits was written by the forward kernel; it is scaled by the upstream gradient in place (the kernel
+    returns at once when that is 1, the usual case) and handed on without a copy, so a graph can be walked once."""
+    if dloss is None:
+        return None, None, None
+    if ctx.dlogits_consumed:
+        raise RuntimeError("maltos::ce_fwd_bwd: backward ran twice through the same loss; its logits gradient is "
+                           "scaled in place by the first pass, so recompute the loss instead of retaining the graph")
     (dlogits,) = ctx.saved_tensors
-    return torch.ops.maltos.scale_by_scalar(dlogits, dloss), None, None
+    torch.ops.maltos.scale_by_scalar_(dlogits, dloss)
+    ctx.dlogits_consumed = True
+    return dlogits, None, None
 
 
 torch.library.register_autograd("maltos::ce_fwd_bwd", _ce_backward, setup_context=_ce_setup)
@@ -550,6 +576,23 @@ def scale_(x: torch.Tensor, scale: float) -> torch.Tensor:
     _flat_f32(x, "x")
     _lib.check(_lib.lib().mlts_scale(_p(x), float(scale), x.numel(), _stream()))
     return x
+
+
+def grad_sum_slices(parts: torch.Tensor, out: torch.Tensor | None = None, *, accumulate: bool = False) -> torch.Tensor:
+    """parts [slices, ...] -> sum over the slices, added in fp32 and rounded once; with `out` the result is written
+    there (accumulate=True: added onto what `out` holds)."""
+    _require_gpu(parts, out)
+    if parts.dim() < 2 or not parts.is_contiguous():
+        raise ValueError("parts must be a contiguous tensor [slices, ...]")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate=True needs an output tensor")
+        out = torch.empty(parts.shape[1:], dtype=parts.dtype, device=parts.device)
+    elif out.dtype != parts.dtype or out.shape != parts.shape[1:] or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the dtype and the per-slice shape of parts")
+    _lib.check(_lib.lib().mlts_grad_sum_slices(_p(out), _p(parts), _dtype_code(parts), parts.size(0), out.numel(),
+                                               int(accumulate), _stream()))
+    return out
 
 
 def grad_to_f32_(dst: torch.Tensor, src: torch.Tensor, *, accumulate: bool = False,

@@ -130,6 +130,25 @@ def test_cross_entropy(dev, dtype, rows, vocab):
     assert abs(loss.item() - lib.item()) <= 1e-4 * abs(lib.item()) + 1e-6
 
 
+def test_cross_entropy_backward_consumes_its_buffer_once(dev):
+    """The logits gradient written by the forward kernel is scaled in place and handed on without a copy: the result
+    is right for a scaled loss, nothing of the logits' size is allocated in backward, and a second walk is refused."""
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(16, 1000, generator=g)
+    labels = torch.randint(0, 1000, (16,), generator=g)
+    lg = logits.to(dev).requires_grad_(True)
+    loss = ops.cross_entropy(lg, labels.to(dev))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    (loss * 0.5).backward(retain_graph=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() - before < 2 * lg.numel() * 4     # lg.grad itself, no second buffer
+    _, want_grad = ol.causal_cross_entropy_explicit(logits, labels)
+    assert torch.allclose(lg.grad.cpu(), 0.5 * want_grad, rtol=1e-5, atol=1e-8)
+    with pytest.raises(RuntimeError, match="backward ran twice"):
+        loss.backward()
+
+
 def test_cross_entropy_without_targets_is_zero(dev):
     lg = torch.randn(2, 3, 5, device=dev, requires_grad=True)
     loss = ops.cross_entropy(lg, torch.full((2, 3), -100, device=dev))

@@ -176,3 +176,69 @@ def test_zero1_flat_buffers_step_equals_plain_optimizer(dev, dtype):
         for p, q in zip(zero_model.parameters(), plain_model.parameters()):
             assert p.data_ptr() >= z.data_buffer.data_ptr()  # still a view of the flat buffer
             torch.testing.assert_close(p.detach().float(), q.detach().float(), rtol=1e-5 if dtype == torch.float32 else 2 ** -7, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("slices,shape", [(1, (7,)), (4, (33, 65)), (16, (512, 512)), (8, (3, 1376))])
+def test_grad_sum_slices(dev, dtype, slices, shape):
+    """Sum of the row-slice partial products in fp32 with one rounding, plain and added onto an existing gradient
+    (vector path, odd sizes and the one-slice case)."""
+    from maltos_amd import ops
+
+    g = torch.Generator().manual_seed(slices * 131 + len(shape))
+    parts = torch.randn(slices, *shape, generator=g).to(dtype)
+    old = torch.randn(*shape, generator=g).to(dtype)
+    got = ops.grad_sum_slices(parts.to(dev))
+    want = parts.double().sum(0)
+    # one final rounding to dtype plus, in fp32, one rounding per term of the running sum
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else (slices + 1) * 2.0 ** -24
+    assert got.dtype == dtype and got.shape == tuple(shape)
+    mag = parts.double().abs().sum(0)      # rounding of the running fp32 sum scales with the terms, not with the result
+    assert ((got.double().cpu() - want).abs() <= ulp * mag + 1e-9).all()
+    acc = old.to(dev).clone()
+    assert ops.grad_sum_slices(parts.to(dev), acc, accumulate=True) is acc
+    want_acc = want + old.double()
+    assert ((acc.double().cpu() - want_acc).abs() <= ulp * (mag + old.double().abs()) + 1e-9).all()
+    with pytest.raises(ValueError):
+        ops.grad_sum_slices(parts.to(dev), accumulate=True)
+    with pytest.raises(ValueError):
+        ops.grad_sum_slices(parts.to(dev), torch.empty(3, device=dev, dtype=dtype))
+
+
+@pytest.mark.parametrize("rows,out_f,in_f", [(4096, 256, 256), (512, 64, 96)])
+def test_linear_accumulates_weight_grad_into_bound_buffer(dev, rows, out_f, in_f):
+    """HipLinear with accumulate_into_grad adds dW into the existing gradient buffer (sliced and single-product
+    forms) and leaves the same numbers as autograd's own accumulation, to one bf16 rounding."""
+    from maltos_amd.llama import HipLinear, _weight_grad_splits
+
+    assert (_weight_grad_splits(rows, out_f, in_f) > 1) == (rows == 4096)
+    torch.manual_seed(3)
+    plain = HipLinear(in_f, out_f, bias=False).to(dev).to(torch.bfloat16)
+    fused = HipLinear(in_f, out_f, bias=False).to(dev).to(torch.bfloat16)
+    fused.load_state_dict(plain.state_dict())
+    fused.accumulate_into_grad = True
+    start = (torch.randn(out_f, in_f, device=dev) * 0.5).to(torch.bfloat16)
+    plain.weight.grad = start.clone()
+    fused.weight.grad = start.clone()
+    buffer_ptr = fused.weight.grad.data_ptr()
+    x = torch.randn(rows, in_f, device=dev).to(torch.bfloat16)
+    dy = (torch.randn(rows, out_f, device=dev) * 0.1).to(torch.bfloat16)
+    grads = []
+    for lin in (plain, fused):
+        xi = x.clone().requires_grad_(True)
+        lin(xi).backward(dy)
+        grads.append(xi.grad)
+    assert fused.weight.grad.data_ptr() == buffer_ptr
+    assert torch.equal(grads[0], grads[1])
+    exact = start.double() + dy.double().t() @ x.double()
+    # both forms carry the bf16 rounding of the GEMM outputs; the fused one saves the rounding of `grad += dW`
+    err_plain = (plain.weight.grad.double() - exact).abs()
+    err_fused = (fused.weight.grad.double() - exact).abs()
+    bound = 2.0 ** -7 * exact.abs().max()      # the partial products are of the size of the largest results
+    assert err_plain.max() <= bound and err_fused.max() <= bound
+    assert err_fused.mean() <= err_plain.mean() * 1.02
+    # without a bound gradient the module falls back to returning dW
+    fused.weight.grad = None
+    xi = x.clone().requires_grad_(True)
+    fused(xi).backward(dy)
+    assert fused.weight.grad is not None and (fused.weight.grad.double() - (exact - start.double())).abs().max() < 0.5
