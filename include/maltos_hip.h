@@ -128,6 +128,17 @@ int64_t mlts_rmsnorm_bwd_workspace_bytes(int64_t rows, int32_t hidden);
 int mlts_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw,
                      void* workspace, int64_t workspace_bytes, int64_t rows, int32_t hidden, int32_t dtype,
                      mlts_stream_t stream);
+/* The residual add in front of a norm fused into it (models/llama.py:224-230 `x = x + sublayer(...)` followed by the
+ * next RMSNorm, :55-57): sum_out = round(x + res), y = RMSNorm(sum_out) with the roundings of the two separate ops.
+ * sum_out and y are different buffers; sum_out may alias x or res. */
+int mlts_add_rmsnorm_fwd(const void* x, const void* res, void* sum_out, const void* w, void* y, float* rstd_out,
+                         int64_t rows, int32_t hidden, float eps, int32_t dtype, mlts_stream_t stream);
+/* Backward of the pair: x is the summed row (sum_out above), dres the gradient reaching it by the residual path;
+ * dx = round(dx of the norm) + dres, the gradient of both addends.  Other arguments as mlts_rmsnorm_bwd. */
+int mlts_add_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
+                         void* dw, void* workspace, int64_t workspace_bytes, int64_t rows, int32_t hidden, int32_t dtype,
+                         mlts_stream_t stream);
+
 
 /* Interleaved-pair rotary embedding (models/llama.py:89-94,134-144):
  *   (x[2i], x[2i+1]) -> (x[2i] c - x[2i+1] s, x[2i] s + x[2i+1] c), c/s = cos/sin[pos, i],

@@ -79,6 +79,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_rmsnorm_fwd": (C.c_int, [_P, _P, _P, _P, C.c_int64, C.c_int32, C.c_float, C.c_int32, _P]),
     "mlts_rmsnorm_bwd_workspace_bytes": (C.c_int64, [C.c_int64, C.c_int32]),
     "mlts_rmsnorm_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int32, C.c_int32, _P]),
+    "mlts_add_rmsnorm_fwd": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int32, C.c_float, C.c_int32, _P]),
+    "mlts_add_rmsnorm_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int32, C.c_int32, _P]),
     "mlts_rope": (
         C.c_int,
         [_P, _I64P, _P, _I64P, _P, _P, C.c_int32, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,

@@ -16,20 +16,32 @@ constexpr int kWaves = kThreads / MLTS_WAVE;
 
 // ============================== RMSNorm ==================================================
 // One wavefront per row; a row is walked in chunks of 64 lanes x 16 bytes.
-template <typename T>
-__global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+// ADD: the normalised row is h = x + res, rounded to T as the eager residual add rounds it; h is stored to `sum_out`
+// (which the second pass reads back: a lane reads only what it wrote itself) and is the row the statistics are of.
+template <typename T, bool ADD>
+__global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ res,
+                                                               T* __restrict__ sum_out, const T* __restrict__ w,
                                                                T* __restrict__ y, float* __restrict__ rstd_out,
                                                                int64_t rows, int hidden, float eps) {
   constexpr int N = Vec16<T>::N;
   const int lane = threadIdx.x & (MLTS_WAVE - 1);
   const int64_t row = static_cast<int64_t>(blockIdx.x) * kWaves + (threadIdx.x / MLTS_WAVE);
   if (row >= rows) return;
-  const T* xr = x + row * hidden;
+  const T* xr = ADD ? sum_out + row * hidden : x + row * hidden;
   T* yr = y + row * hidden;
   const int nvec = hidden / N;
   float ss = 0.f;
   for (int c = lane; c < nvec; c += MLTS_WAVE) {
-    Vec16<T> t = reinterpret_cast<const Vec16<T>*>(xr)[c];
+    Vec16<T> t;
+    if (ADD) {
+      const Vec16<T> a = reinterpret_cast<const Vec16<T>*>(x + row * hidden)[c];
+      const Vec16<T> b = reinterpret_cast<const Vec16<T>*>(res + row * hidden)[c];
+#pragma unroll
+      for (int j = 0; j < N; ++j) t.set(j, a.get(j) + b.get(j));
+      reinterpret_cast<Vec16<T>*>(sum_out + row * hidden)[c] = t;
+    } else {
+      t = reinterpret_cast<const Vec16<T>*>(xr)[c];
+    }
 #pragma unroll
     for (int j = 0; j < N; ++j) {
       float f = t.get(j);
@@ -60,9 +72,12 @@ constexpr int kMaxChunks = 8;
 
 // CH = 16-byte chunks per lane and row (1, 2, 4 or 8); 8 / CH rows of a wavefront are in flight at once and their
 // vectors stay in registers between the two passes (one row at a time leaves the memory latency of every row exposed).
-template <typename T, int CH>
+// dres (may be null): gradient that reaches the same row by the residual path; dx = round(dx_norm) + dres, the two
+// roundings of autograd's own sum of the two paths.
+template <typename T, int CH, bool RES>
 __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                                                                const T* __restrict__ w, const float* __restrict__ rstd,
+                                                               const T* __restrict__ dres,
                                                                T* __restrict__ dx, float* __restrict__ dw_partial,
                                                                int64_t rows, int hidden, int rows_per_block) {
   constexpr int N = Vec16<T>::N;
@@ -87,7 +102,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restri
   if (row_end > rows) row_end = rows;
   const float inv_h = 1.0f / static_cast<float>(hidden);
   for (int64_t row = row0 + wave; row < row_end; row += kWaves * R) {
-    Vec16<T> xv[R][CH], dv[R][CH];
+    Vec16<T> xv[R][CH], dv[R][CH], rv[RES ? R : 1][CH];
     float rr[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
@@ -100,6 +115,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restri
         if (col < nvec) {
           xv[i][c] = reinterpret_cast<const Vec16<T>*>(x + ri * hidden)[col];
           dv[i][c] = reinterpret_cast<const Vec16<T>*>(dy + ri * hidden)[col];
+          if (RES) rv[RES ? i : 0][c] = reinterpret_cast<const Vec16<T>*>(dres + ri * hidden)[col];
         }
       }
     }
@@ -132,7 +148,8 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restri
 #pragma unroll
             for (int j = 0; j < N; ++j) {
               float xh = xv[i][c].get(j) * r;
-              o.set(j, r * (dv[i][c].get(j) * wv[c].get(j) - xh * dot));
+              const float g = r * (dv[i][c].get(j) * wv[c].get(j) - xh * dot);
+              o.set(j, RES ? round_to<T>(g) + rv[RES ? i : 0][c].get(j) : g);
             }
             reinterpret_cast<Vec16<T>*>(dxr)[col] = o;
           }
@@ -314,32 +331,44 @@ int stream_grid(int64_t nvec) {
 }
 
 template <typename T>
-int rmsnorm_fwd_t(const void* x, const void* w, void* y, float* rstd, int64_t rows, int hidden, float eps,
-                  hipStream_t st) {
+int rmsnorm_fwd_t(const void* x, const void* res, void* sum_out, const void* w, void* y, float* rstd, int64_t rows,
+                  int hidden, float eps, hipStream_t st) {
   const int64_t blocks = (rows + kWaves - 1) / kWaves;
   MltsKernelTimer timer("rmsnorm_fwd", st);
-  hipLaunchKernelGGL(rmsnorm_fwd_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
-                     static_cast<const T*>(w), static_cast<T*>(y), rstd, rows, hidden, eps);
+  if (res)
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
+                       static_cast<const T*>(res), static_cast<T*>(sum_out), static_cast<const T*>(w), static_cast<T*>(y),
+                       rstd, rows, hidden, eps);
+  else
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<T, false>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
+                       static_cast<const T*>(nullptr), static_cast<T*>(nullptr), static_cast<const T*>(w),
+                       static_cast<T*>(y), rstd, rows, hidden, eps);
   return mlts_check_launch("mlts_rmsnorm_fwd");
 }
 
 template <typename T>
-int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw, float* partial,
-                  int64_t rows, int hidden, hipStream_t st) {
+int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx, void* dw,
+                  float* partial, int64_t rows, int hidden, hipStream_t st) {
   const int blocks = rmsnorm_bwd_blocks(rows);
   const int rows_per_block = static_cast<int>((rows + blocks - 1) / blocks);
   const size_t smem = static_cast<size_t>(kWaves) * hidden * sizeof(float);
   MltsKernelTimer timer("rmsnorm_bwd", st);
   const int chunks = (hidden / Vec16<T>::N + MLTS_WAVE - 1) / MLTS_WAVE;  // <= kMaxChunks, checked by the caller
-#define MLTS_RMS_BWD(CH)                                                                                              \
-  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH>), dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy), \
-                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<T*>(dx), partial, rows,   \
-                     hidden, rows_per_block)
+#define MLTS_RMS_BWD_RES(CH, RES)                                                                                          \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH, RES>), dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy), \
+                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<const T*>(dres),               \
+                     static_cast<T*>(dx), partial, rows, hidden, rows_per_block)
+#define MLTS_RMS_BWD(CH)             \
+  do {                               \
+    if (dres) MLTS_RMS_BWD_RES(CH, true); \
+    else MLTS_RMS_BWD_RES(CH, false);     \
+  } while (0)
   if (chunks <= 1) MLTS_RMS_BWD(1);
   else if (chunks <= 2) MLTS_RMS_BWD(2);
   else if (chunks <= 4) MLTS_RMS_BWD(4);
   else MLTS_RMS_BWD(8);
 #undef MLTS_RMS_BWD
+#undef MLTS_RMS_BWD_RES
   hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + 31) / 32), dim3(kThreads), 0, st,
                      partial, blocks, hidden, static_cast<T*>(dw));
   return mlts_check_launch("mlts_rmsnorm_bwd");
@@ -407,43 +436,76 @@ inline bool known_dtype(int dtype) { return dtype == MLTS_BF16 || dtype == MLTS_
 
 }  // namespace
 
+namespace {
+int rmsnorm_fwd_checked(const char* who, const void* x, const void* res, void* sum_out, const void* w, void* y,
+                        float* rstd_out, int64_t rows, int32_t hidden, float eps, int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  MLTS_REQUIRE(rows >= 0 && hidden > 0, "%s: bad shape rows=%lld hidden=%d", who, (long long)rows, hidden);
+  MLTS_REQUIRE(hidden % elem_per_vec(dtype) == 0, "%s: hidden=%d must be a multiple of %d", who, hidden, elem_per_vec(dtype));
+  if (rows == 0) return MLTS_OK;
+  MLTS_REQUIRE(x && w && y, "%s: null pointer", who);
+  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(y), "%s: pointers must be 16-byte aligned", who);
+  if (res) {
+    MLTS_REQUIRE(sum_out, "%s: null pointer", who);
+    MLTS_REQUIRE(mlts_aligned16(res) && mlts_aligned16(sum_out), "%s: pointers must be 16-byte aligned", who);
+    MLTS_REQUIRE(sum_out != y, "%s: sum_out and y must be different buffers", who);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? rmsnorm_fwd_t<bf16_t>(x, res, sum_out, w, y, rstd_out, rows, hidden, eps, st)
+                            : rmsnorm_fwd_t<float>(x, res, sum_out, w, y, rstd_out, rows, hidden, eps, st);
+}
+}  // namespace
+
 extern "C" int mlts_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd_out, int64_t rows, int32_t hidden,
                                 float eps, int32_t dtype, mlts_stream_t stream) {
-  MLTS_REQUIRE(known_dtype(dtype), "mlts_rmsnorm_fwd: unknown dtype %d", dtype);
-  MLTS_REQUIRE(rows >= 0 && hidden > 0, "mlts_rmsnorm_fwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
-  MLTS_REQUIRE(hidden % elem_per_vec(dtype) == 0, "mlts_rmsnorm_fwd: hidden=%d must be a multiple of %d", hidden,
-               elem_per_vec(dtype));
-  if (rows == 0) return MLTS_OK;
-  MLTS_REQUIRE(x && w && y, "mlts_rmsnorm_fwd: null pointer");
-  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(y), "mlts_rmsnorm_fwd: pointers must be 16-byte aligned");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  return dtype == MLTS_BF16 ? rmsnorm_fwd_t<bf16_t>(x, w, y, rstd_out, rows, hidden, eps, st)
-                            : rmsnorm_fwd_t<float>(x, w, y, rstd_out, rows, hidden, eps, st);
+  return rmsnorm_fwd_checked("mlts_rmsnorm_fwd", x, nullptr, nullptr, w, y, rstd_out, rows, hidden, eps, dtype, stream);
+}
+
+extern "C" int mlts_add_rmsnorm_fwd(const void* x, const void* res, void* sum_out, const void* w, void* y, float* rstd_out,
+                                    int64_t rows, int32_t hidden, float eps, int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(rows == 0 || res, "mlts_add_rmsnorm_fwd: null pointer");
+  return rmsnorm_fwd_checked("mlts_add_rmsnorm_fwd", x, res, sum_out, w, y, rstd_out, rows, hidden, eps, dtype, stream);
 }
 
 extern "C" int64_t mlts_rmsnorm_bwd_workspace_bytes(int64_t rows, int32_t hidden) {
   return static_cast<int64_t>(rmsnorm_bwd_blocks(rows)) * hidden * static_cast<int64_t>(sizeof(float));
 }
 
+namespace {
+int rmsnorm_bwd_checked(const char* who, const void* dy, const void* x, const void* w, const float* rstd, const void* dres,
+                        void* dx, void* dw, void* workspace, int64_t workspace_bytes, int64_t rows, int32_t hidden,
+                        int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(known_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  MLTS_REQUIRE(rows > 0 && hidden > 0, "%s: bad shape rows=%lld hidden=%d", who, (long long)rows, hidden);
+  const int n = elem_per_vec(dtype);
+  MLTS_REQUIRE(hidden % n == 0, "%s: hidden=%d must be a multiple of %d", who, hidden, n);
+  MLTS_REQUIRE(hidden <= MLTS_WAVE * n * kMaxChunks, "%s: hidden=%d exceeds the supported maximum %d", who, hidden,
+               MLTS_WAVE * n * kMaxChunks);
+  MLTS_REQUIRE(dy && x && w && rstd && dx && dw && workspace, "%s: null pointer", who);
+  MLTS_REQUIRE(mlts_aligned16(dy) && mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(dx) && mlts_aligned16(dres),
+               "%s: pointers must be 16-byte aligned", who);
+  MLTS_REQUIRE(workspace_bytes >= mlts_rmsnorm_bwd_workspace_bytes(rows, hidden), "%s: workspace too small (%lld < %lld)",
+               who, (long long)workspace_bytes, (long long)mlts_rmsnorm_bwd_workspace_bytes(rows, hidden));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* partial = static_cast<float*>(workspace);
+  return dtype == MLTS_BF16 ? rmsnorm_bwd_t<bf16_t>(dy, x, w, rstd, dres, dx, dw, partial, rows, hidden, st)
+                            : rmsnorm_bwd_t<float>(dy, x, w, rstd, dres, dx, dw, partial, rows, hidden, st);
+}
+}  // namespace
+
 extern "C" int mlts_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw,
                                 void* workspace, int64_t workspace_bytes, int64_t rows, int32_t hidden, int32_t dtype,
                                 mlts_stream_t stream) {
-  MLTS_REQUIRE(known_dtype(dtype), "mlts_rmsnorm_bwd: unknown dtype %d", dtype);
-  MLTS_REQUIRE(rows > 0 && hidden > 0, "mlts_rmsnorm_bwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
-  const int n = elem_per_vec(dtype);
-  MLTS_REQUIRE(hidden % n == 0, "mlts_rmsnorm_bwd: hidden=%d must be a multiple of %d", hidden, n);
-  MLTS_REQUIRE(hidden <= MLTS_WAVE * n * kMaxChunks, "mlts_rmsnorm_bwd: hidden=%d exceeds the supported maximum %d",
-               hidden, MLTS_WAVE * n * kMaxChunks);
-  MLTS_REQUIRE(dy && x && w && rstd && dx && dw && workspace, "mlts_rmsnorm_bwd: null pointer");
-  MLTS_REQUIRE(mlts_aligned16(dy) && mlts_aligned16(x) && mlts_aligned16(w) && mlts_aligned16(dx),
-               "mlts_rmsnorm_bwd: pointers must be 16-byte aligned");
-  MLTS_REQUIRE(workspace_bytes >= mlts_rmsnorm_bwd_workspace_bytes(rows, hidden),
-               "mlts_rmsnorm_bwd: workspace too small (%lld < %lld)", (long long)workspace_bytes,
-               (long long)mlts_rmsnorm_bwd_workspace_bytes(rows, hidden));
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  float* partial = static_cast<float*>(workspace);
-  return dtype == MLTS_BF16 ? rmsnorm_bwd_t<bf16_t>(dy, x, w, rstd, dx, dw, partial, rows, hidden, st)
-                            : rmsnorm_bwd_t<float>(dy, x, w, rstd, dx, dw, partial, rows, hidden, st);
+  return rmsnorm_bwd_checked("mlts_rmsnorm_bwd", dy, x, w, rstd, nullptr, dx, dw, workspace, workspace_bytes, rows, hidden,
+                             dtype, stream);
+}
+
+extern "C" int mlts_add_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres,
+                                    void* dx, void* dw, void* workspace, int64_t workspace_bytes, int64_t rows,
+                                    int32_t hidden, int32_t dtype, mlts_stream_t stream) {
+  MLTS_REQUIRE(dres, "mlts_add_rmsnorm_bwd: null pointer");
+  return rmsnorm_bwd_checked("mlts_add_rmsnorm_bwd", dy, x, w, rstd, dres, dx, dw, workspace, workspace_bytes, rows,
+                             hidden, dtype, stream);
 }
 
 extern "C" int mlts_rope(const void* x, const int64_t x_stride[3], void* y, const int64_t y_stride[3],

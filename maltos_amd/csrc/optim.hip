@@ -326,27 +326,34 @@ template <typename T, bool ACC>
 __global__ __launch_bounds__(kThreads) void grad_sum_slices_vec_kernel(T* __restrict__ out, const T* __restrict__ parts, int slices,
                                                                        int64_t nvec) {
   using V = Vec16<T>;
+  constexpr int U = 8;  // slice loads in flight per lane: the buffers are small, so latency, not bandwidth, is the limit
   const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
   const V* pv = reinterpret_cast<const V*>(parts);
   V* ov = reinterpret_cast<V*>(out);
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < nvec; i += stride) {
     float acc[V::N];
-    if (ACC) {
-      const V o = ov[i];
+    V o;
+    if (ACC) o = ov[i];
 #pragma unroll
-      for (int j = 0; j < V::N; ++j) acc[j] = o.get(j);
-    } else {
+    for (int j = 0; j < V::N; ++j) acc[j] = 0.f;
+    int s = 0;
+    for (; s + U <= slices; s += U) {
+      V p[U];
 #pragma unroll
-      for (int j = 0; j < V::N; ++j) acc[j] = 0.f;
+      for (int u = 0; u < U; ++u) p[u] = pv[static_cast<int64_t>(s + u) * nvec + i];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int j = 0; j < V::N; ++j) acc[j] += p[u].get(j);
     }
-    for (int s = 0; s < slices; ++s) {
+    for (; s < slices; ++s) {
       const V p = pv[static_cast<int64_t>(s) * nvec + i];
 #pragma unroll
       for (int j = 0; j < V::N; ++j) acc[j] += p.get(j);
     }
     V r;
 #pragma unroll
-    for (int j = 0; j < V::N; ++j) r.set(j, acc[j]);
+    for (int j = 0; j < V::N; ++j) r.set(j, ACC ? acc[j] + o.get(j) : acc[j]);
     ov[i] = r;
   }
 }
@@ -368,7 +375,7 @@ void launch_grad_sum_slices(void* out, const void* parts, int slices, int64_t n,
   const T* p = static_cast<const T*>(parts);
   if (n % N == 0 && mlts_aligned16(out) && mlts_aligned16(parts)) {
     const int64_t nvec = n / N;
-    const int blocks = grid_for(nvec, 4096);
+    const int blocks = grid_for(nvec, 8192);
     if (acc)
       hipLaunchKernelGGL((grad_sum_slices_vec_kernel<T, true>), dim3(blocks), dim3(kThreads), 0, st, o, p, slices, nvec);
     else

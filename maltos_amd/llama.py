@@ -36,6 +36,9 @@ class LlamaConfig:
     rope_theta: float = 10000.0
     tie_word_embeddings: bool = False
     attention_backend: str = AttentionBackend.HIP
+    # each residual add is done inside the RMSNorm kernel that follows it (same values; one pass less per sublayer,
+    # forward and backward); False keeps the reference's op sequence
+    fuse_residual_norm: bool = True
 
     def __post_init__(self) -> None:
         validate_attention_backend(self.attention_backend)
@@ -220,10 +223,24 @@ class LlamaDecoderLayer(nn.Module):
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
 
     def forward(self, x: torch.Tensor, position_offset: int = 0, position_ids: torch.Tensor | None = None,
-                sequence_ids: torch.Tensor | None = None) -> torch.Tensor:
-        x = x + self.self_attn(self.input_layernorm(x), position_offset=position_offset, position_ids=position_ids,
-                               sequence_ids=sequence_ids)
-        return x + self.mlp(self.post_attention_layernorm(x))
+                sequence_ids: torch.Tensor | None = None, pending: torch.Tensor | None = None,
+                defer_residual: bool = False):
+        """Reference form (:217-231): x -> x.  With `defer_residual` the layer returns (x, mlp_out) and leaves the last
+        residual add to whoever normalises next, and takes such a not-yet-added `pending` from the layer before."""
+        if not defer_residual:
+            if pending is not None:
+                x = x + pending
+            x = x + self.self_attn(self.input_layernorm(x), position_offset=position_offset, position_ids=position_ids,
+                                   sequence_ids=sequence_ids)
+            return x + self.mlp(self.post_attention_layernorm(x))
+        ln1, ln2 = self.input_layernorm, self.post_attention_layernorm
+        if pending is None:
+            normed = ln1(x)
+        else:
+            x, normed = ops.add_rms_norm(x, pending, ln1.weight, ln1.eps)
+        attn_out = self.self_attn(normed, position_offset=position_offset, position_ids=position_ids, sequence_ids=sequence_ids)
+        x, normed = ops.add_rms_norm(x, attn_out, ln2.weight, ln2.eps)
+        return x, self.mlp(normed)
 
 
 class LlamaForCausalLM(nn.Module):
@@ -260,9 +277,17 @@ class LlamaForCausalLM(nn.Module):
             raise ValueError("LlamaForCausalLM requires input_ids or hidden_states")
         else:
             x = self.embed_tokens(input_ids)
-        for layer in self.layers:
-            x = layer(x, position_offset=position_offset, position_ids=position_ids, sequence_ids=sequence_ids)
-        logits = self.lm_head(self.norm(x))
+        if self.config.fuse_residual_norm and x.is_cuda and len(self.layers) > 0:
+            pending = None
+            for layer in self.layers:
+                x, pending = layer(x, position_offset=position_offset, position_ids=position_ids, sequence_ids=sequence_ids,
+                                   pending=pending, defer_residual=True)
+            _, normed = ops.add_rms_norm(x, pending, self.norm.weight, self.norm.eps)
+        else:
+            for layer in self.layers:
+                x = layer(x, position_offset=position_offset, position_ids=position_ids, sequence_ids=sequence_ids)
+            normed = self.norm(x)
+        logits = self.lm_head(normed)
         if labels is None:
             return logits
         if input_ids is not None and labels.shape != input_ids.shape:

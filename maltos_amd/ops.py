@@ -231,6 +231,41 @@ def _rmsnorm_bwd(dy, x, w, rstd):
     return dx.view(x.shape), dw
 
 
+def _add_rmsnorm_fwd(x, res, w, eps):
+    _require_gpu(x, res, w)
+    hidden = x.size(-1)
+    if w.shape != (hidden,) or w.dtype != x.dtype:
+        raise ValueError("RMSNorm weight must be [hidden] with the dtype of x")
+    if res.shape != x.shape or res.dtype != x.dtype:
+        raise ValueError("the residual must have the shape and dtype of x")
+    x2 = x.contiguous().view(-1, hidden)
+    r2 = res.contiguous().view(-1, hidden)
+    h = torch.empty_like(x2)
+    y = torch.empty_like(x2)
+    rstd = torch.empty(x2.size(0), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().mlts_add_rmsnorm_fwd(_p(x2), _p(r2), _p(h), _p(w.contiguous()), _p(y), _p(rstd), x2.size(0), hidden,
+                                               float(eps), _dtype_code(x), _stream()))
+    return h.view(x.shape), y.view(x.shape), rstd
+
+
+def _add_rmsnorm_bwd(dy, dres, h, w, rstd):
+    _require_gpu(dy, dres, h, w, rstd)
+    hidden = h.size(-1)
+    h2 = h.contiguous().view(-1, hidden)
+    dy2 = dy.contiguous().view(-1, hidden)
+    dr2 = dres.contiguous().view(-1, hidden)
+    dx = torch.empty_like(h2)
+    dw = torch.empty_like(w)
+    if h2.size(0) == 0:
+        return dx.view(h.shape), dw.zero_()
+    L = _lib.lib()
+    ws_bytes = L.mlts_rmsnorm_bwd_workspace_bytes(h2.size(0), hidden)
+    ws = _workspace(ws_bytes, h.device)
+    _lib.check(L.mlts_add_rmsnorm_bwd(_p(dy2), _p(h2), _p(w.contiguous()), _p(rstd), _p(dr2), _p(dx), _p(dw), _p(ws), ws_bytes,
+                                      h2.size(0), hidden, _dtype_code(h), _stream()))
+    return dx.view(h.shape), dw
+
+
 def _rope(x, cos, sin, positions, position_offset, inverse):
     _require_gpu(x, cos, sin, positions)
     if x.dim() != 4:
@@ -299,6 +334,8 @@ _LIBRARY.define(
 )
 _LIBRARY.define("rmsnorm_fwd(Tensor x, Tensor w, float eps) -> (Tensor, Tensor)")
 _LIBRARY.define("rmsnorm_bwd(Tensor dy, Tensor x, Tensor w, Tensor rstd) -> (Tensor, Tensor)")
+_LIBRARY.define("add_rmsnorm_fwd(Tensor x, Tensor res, Tensor w, float eps) -> (Tensor, Tensor, Tensor)")
+_LIBRARY.define("add_rmsnorm_bwd(Tensor dy, Tensor dres, Tensor h, Tensor w, Tensor rstd) -> (Tensor, Tensor)")
 _LIBRARY.define("rope(Tensor x, Tensor cos, Tensor sin, Tensor? positions, int position_offset, bool inverse) -> Tensor")
 _LIBRARY.define("swiglu_fwd(Tensor gate, Tensor up) -> Tensor")
 _LIBRARY.define("swiglu_bwd(Tensor dh, Tensor gate, Tensor up) -> (Tensor, Tensor)")
@@ -322,7 +359,7 @@ def _cpu_refusal(name: str) -> None:
     _LIBRARY.impl(name, refuse, "CPU")
 
 
-for _name in ("attn_fwd", "attn_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "ce_fwd_bwd",
+for _name in ("attn_fwd", "attn_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "add_rmsnorm_fwd", "add_rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "ce_fwd_bwd",
               "scale_by_scalar", "scale_by_scalar_"):
     _cpu_refusal(_name)
 
@@ -340,6 +377,8 @@ def _attn_bwd_op(dout, q, k, v, o, lse, mask_mode, scale, q_pos, k_pos, q_seq, k
 
 _impl("rmsnorm_fwd")(_rmsnorm_fwd)
 _impl("rmsnorm_bwd")(_rmsnorm_bwd)
+_impl("add_rmsnorm_fwd")(_add_rmsnorm_fwd)
+_impl("add_rmsnorm_bwd")(_add_rmsnorm_bwd)
 _impl("rope")(_rope)
 _impl("swiglu_fwd")(_swiglu_fwd)
 _impl("swiglu_bwd")(_swiglu_bwd)
@@ -388,6 +427,17 @@ def _(x, w, eps):
 @torch.library.register_fake("maltos::rmsnorm_bwd")
 def _(dy, x, w, rstd):
     return torch.empty_like(x), torch.empty_like(w)
+
+
+@torch.library.register_fake("maltos::add_rmsnorm_fwd")
+def _(x, res, w, eps):
+    return (torch.empty_like(x), torch.empty_like(x),
+            x.new_empty((x.numel() // max(1, x.size(-1)),), dtype=torch.float32))
+
+
+@torch.library.register_fake("maltos::add_rmsnorm_bwd")
+def _(dy, dres, h, w, rstd):
+    return torch.empty_like(h), torch.empty_like(w)
 
 
 @torch.library.register_fake("maltos::rope")
@@ -454,6 +504,28 @@ def _rms_backward(ctx, dy, _drstd):
 torch.library.register_autograd("maltos::rmsnorm_fwd", _rms_backward, setup_context=_rms_setup)
 
 
+def _add_rms_setup(ctx, inputs, output):
+    _x, _res, w, _eps = inputs
+    ctx.save_for_backward(output[0], w, output[2])
+    ctx.set_materialize_grads(False)
+
+
+def _add_rms_backward(ctx, dh, dy, _drstd):
+    """dh: gradient of the summed row from its later uses (the residual path), dy: gradient of the normalised row.
+    Both addends receive the same gradient."""
+    h, w, rstd = ctx.saved_tensors
+    if dy is None:
+        return dh, dh, None, None
+    if dh is None:
+        dx, dw = torch.ops.maltos.rmsnorm_bwd(dy, h, w, rstd)
+    else:
+        dx, dw = torch.ops.maltos.add_rmsnorm_bwd(dy, dh, h, w, rstd)
+    return dx, dx, dw, None
+
+
+torch.library.register_autograd("maltos::add_rmsnorm_fwd", _add_rms_backward, setup_context=_add_rms_setup)
+
+
 def _rope_setup(ctx, inputs, output):
     _x, cos, sin, positions, position_offset, inverse = inputs
     ctx.save_for_backward(cos, sin, positions)
@@ -518,6 +590,12 @@ def attention(q, k, v, *, mask_mode: int = MASK_CAUSAL, scale: float | None = No
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return torch.ops.maltos.rmsnorm_fwd(x, weight, float(eps))[0]
+
+
+def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """(h, y) with h = x + residual and y = rms_norm(h), in one pass and with the roundings of the two separate ops."""
+    h, y, _ = torch.ops.maltos.add_rmsnorm_fwd(x, residual, weight, float(eps))
+    return h, y
 
 
 def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, positions: torch.Tensor | None = None,

@@ -100,3 +100,35 @@ def test_capture_refuses_unbound_gradients_and_changed_shapes(dev):
     short = {k: v[:, :32].contiguous() for k, v in batch.items()}
     with pytest.raises(ValueError, match="recorded"):
         step(short)
+
+
+def test_fused_residual_norm_and_in_buffer_gradients_equal_the_plain_model(dev):
+    """The model with residual adds fused into the norms (the default) and with weight gradients accumulated straight
+    into bound buffers gives bit for bit the loss and the gradients of the reference op sequence."""
+    from dataclasses import replace
+
+    from maltos_amd.llama import LlamaForCausalLM, set_grad_accumulation_into_buffers
+
+    cfg, fused_model, _ = _make(dev, torch.bfloat16)
+    plain_model = LlamaForCausalLM(replace(cfg, fuse_residual_norm=False)).to(dev).to(torch.bfloat16)
+    plain_model.load_state_dict(fused_model.state_dict())
+    assert fused_model.config.fuse_residual_norm
+    assert set_grad_accumulation_into_buffers(fused_model) == 2 * 7
+    batch = _batches(cfg, dev, 1)[0]
+    for p in plain_model.parameters():
+        p.grad = None
+    for p in fused_model.parameters():
+        p.grad = torch.zeros_like(p)
+    want = plain_model(batch)
+    want.backward()
+    got = fused_model(batch)
+    got.backward()
+    assert torch.equal(got, want)
+    for (name, p), q in zip(plain_model.named_parameters(), fused_model.parameters()):
+        assert torch.equal(p.grad, q.grad), name
+    # packed documents take the same path
+    packed = dict(batch)
+    S = batch["input_ids"].size(1)
+    packed["position_ids"] = (torch.arange(S, device=dev) % 300).expand_as(batch["input_ids"]).contiguous()
+    packed["sequence_ids"] = (torch.arange(S, device=dev) // 300).expand_as(batch["input_ids"]).contiguous()
+    assert torch.equal(fused_model(packed), plain_model(packed))

@@ -59,6 +59,38 @@ def test_rmsnorm_forward_backward(dev, dtype, rows, hidden):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden", [(1, 256), (37, 512), (300, 1024), (4099, 2048)])
+def test_add_rmsnorm_equals_add_then_rmsnorm(dev, dtype, rows, hidden):
+    """The fused residual add + RMSNorm gives bit for bit what the two separate ops give, forward and backward, with
+    the summed row used again downstream (the residual path) and without."""
+    g = torch.Generator().manual_seed(rows * 7 + hidden)
+    x, res, dy, dh = ((torch.randn(rows, hidden, generator=g)).to(dtype).to(dev) for _ in range(4))
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype).to(dev)
+    for use_residual_path in (True, False):
+        leaves_a = [t.clone().requires_grad_(True) for t in (x, res, w)]
+        h = leaves_a[0] + leaves_a[1]
+        y = ops.rms_norm(h, leaves_a[2], 1e-5)
+        leaves_b = [t.clone().requires_grad_(True) for t in (x, res, w)]
+        h2, y2 = ops.add_rms_norm(leaves_b[0], leaves_b[1], leaves_b[2], 1e-5)
+        assert torch.equal(h, h2) and torch.equal(y, y2)
+        if use_residual_path:
+            torch.autograd.backward([y, h], [dy, dh])
+            torch.autograd.backward([y2, h2], [dy, dh])
+        else:
+            y.backward(dy)
+            y2.backward(dy)
+        for a, b, name in zip(leaves_a, leaves_b, ("x", "res", "w")):
+            assert torch.equal(a.grad, b.grad), (name, use_residual_path)
+    # only the summed row is used: the gradient passes through to both addends
+    xa, ra = x.clone().requires_grad_(True), res.clone().requires_grad_(True)
+    h3, _ = ops.add_rms_norm(xa, ra, w, 1e-5)
+    h3.backward(dh)
+    assert torch.equal(xa.grad, dh) and torch.equal(ra.grad, dh)
+    with pytest.raises(ValueError):
+        ops.add_rms_norm(x, res[:, : hidden // 2], w, 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("use_ids", [False, True])
 def test_rope_forward_backward(dev, dtype, use_ids):
     B, H, S, D = 2, 3, 17, 64
