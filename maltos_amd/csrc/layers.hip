@@ -70,18 +70,21 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_fwd_kernel(const T* __restri
 // partials live in registers (hidden <= 64 * N * kMaxChunks).
 constexpr int kMaxChunks = 8;
 
-// CH = 16-byte chunks per lane and row (1, 2, 4 or 8); 8 / CH rows of a wavefront are in flight at once and their
-// vectors stay in registers between the two passes (one row at a time leaves the memory latency of every row exposed).
+// CH = 16-byte chunks per lane and row (1, 2, 4 or 8); R rows of a wavefront are in flight at once and their vectors
+// stay in registers between the two passes (one row at a time leaves the memory latency of every row exposed); NW
+// wavefronts per block.  A wavefront loads, then computes, then stores, so memory and arithmetic overlap only across
+// wavefronts: narrow rows (CH <= 2) run 16 wavefronts per block, four per SIMD, with correspondingly fewer rows each.
 // dres (may be null): gradient that reaches the same row by the residual path; dx = round(dx_norm) + dres, the two
 // roundings of autograd's own sum of the two paths.
-template <typename T, int CH, bool RES>
-__global__ __launch_bounds__(kThreads) void rmsnorm_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+template <typename T, int CH, bool RES, int R, int NW>
+__global__ __launch_bounds__(NW * MLTS_WAVE) void rmsnorm_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                                                                const T* __restrict__ w, const float* __restrict__ rstd,
                                                                const T* __restrict__ dres,
                                                                T* __restrict__ dx, float* __restrict__ dw_partial,
                                                                int64_t rows, int hidden, int rows_per_block) {
   constexpr int N = Vec16<T>::N;
-  constexpr int R = 8 / CH;
+  constexpr int kWaves = NW;       // shadows the file-wide block shape
+  constexpr int kThreads = NW * MLTS_WAVE;
   extern __shared__ float smem[];  // [kWaves][hidden]
   const int lane = threadIdx.x & (MLTS_WAVE - 1);
   const int wave = threadIdx.x / MLTS_WAVE;
@@ -206,7 +209,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_dw_reduce_kernel(const float
 
 int rmsnorm_bwd_blocks(int64_t rows) {
   int64_t b = (rows + 31) / 32;  // >= 32 rows per block keeps the partial buffer small
-  if (b > 256) b = 256;          // one block per CU; more (tried: 1024) only lengthens the reduction above
+  if (b > 256) b = 256;          // one block per CU: more blocks only lengthen the reduction of their dw partials
   if (b < 1) b = 1;
   return static_cast<int>(b);
 }
@@ -346,29 +349,48 @@ int rmsnorm_fwd_t(const void* x, const void* res, void* sum_out, const void* w, 
   return mlts_check_launch("mlts_rmsnorm_fwd");
 }
 
+template <typename T, int CH, int R, int NW>
+void rmsnorm_bwd_launch(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
+                        float* partial, int64_t rows, int hidden, int blocks, int rows_per_block, hipStream_t st) {
+  const size_t smem = static_cast<size_t>(NW) * hidden * sizeof(float);
+  if (dres)
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH, true, R, NW>), dim3(blocks), dim3(NW * MLTS_WAVE), smem, st,
+                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), rstd,
+                       static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden, rows_per_block);
+  else
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH, false, R, NW>), dim3(blocks), dim3(NW * MLTS_WAVE), smem, st,
+                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), rstd,
+                       static_cast<const T*>(nullptr), static_cast<T*>(dx), partial, rows, hidden, rows_per_block);
+}
+
 template <typename T>
 int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx, void* dw,
                   float* partial, int64_t rows, int hidden, hipStream_t st) {
   const int blocks = rmsnorm_bwd_blocks(rows);
   const int rows_per_block = static_cast<int>((rows + blocks - 1) / blocks);
-  const size_t smem = static_cast<size_t>(kWaves) * hidden * sizeof(float);
   MltsKernelTimer timer("rmsnorm_bwd", st);
   const int chunks = (hidden / Vec16<T>::N + MLTS_WAVE - 1) / MLTS_WAVE;  // <= kMaxChunks, checked by the caller
-#define MLTS_RMS_BWD_RES(CH, RES)                                                                                          \
-  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, CH, RES>), dim3(blocks), dim3(kThreads), smem, st, static_cast<const T*>(dy), \
-                     static_cast<const T*>(x), static_cast<const T*>(w), rstd, static_cast<const T*>(dres),               \
-                     static_cast<T*>(dx), partial, rows, hidden, rows_per_block)
-#define MLTS_RMS_BWD(CH)             \
-  do {                               \
-    if (dres) MLTS_RMS_BWD_RES(CH, true); \
-    else MLTS_RMS_BWD_RES(CH, false);     \
-  } while (0)
-  if (chunks <= 1) MLTS_RMS_BWD(1);
-  else if (chunks <= 2) MLTS_RMS_BWD(2);
-  else if (chunks <= 4) MLTS_RMS_BWD(4);
-  else MLTS_RMS_BWD(8);
+#define MLTS_RMS_BWD(CH, R, NW) \
+  rmsnorm_bwd_launch<T, CH, R, NW>(dy, x, w, rstd, dres, dx, partial, rows, hidden, blocks, rows_per_block, st)
+  if (chunks <= 2) {
+    // rows of one wavefront (of 16 per block) per pass: as many as it has, up to 8 vectors per operand and lane
+    const int per_wave = (rows_per_block + 15) / 16;
+    if (chunks <= 1) {
+      if (per_wave >= 8) MLTS_RMS_BWD(1, 8, 16);
+      else if (per_wave >= 4) MLTS_RMS_BWD(1, 4, 16);
+      else if (per_wave >= 2) MLTS_RMS_BWD(1, 2, 16);
+      else MLTS_RMS_BWD(1, 1, 16);
+    } else {
+      if (per_wave >= 4) MLTS_RMS_BWD(2, 4, 16);
+      else if (per_wave >= 2) MLTS_RMS_BWD(2, 2, 16);
+      else MLTS_RMS_BWD(2, 1, 16);
+    }
+  } else if (chunks <= 4) {
+    MLTS_RMS_BWD(4, 2, 4);
+  } else {
+    MLTS_RMS_BWD(8, 1, 4);
+  }
 #undef MLTS_RMS_BWD
-#undef MLTS_RMS_BWD_RES
   hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<T>, dim3((hidden + 31) / 32), dim3(kThreads), 0, st,
                      partial, blocks, hidden, static_cast<T*>(dw));
   return mlts_check_launch("mlts_rmsnorm_bwd");
