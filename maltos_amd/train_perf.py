@@ -2,6 +2,7 @@
 
     python -m maltos_amd.train_perf --model llama-50m --layout dense  --steps 20 --out summary.json
     python -m maltos_amd.train_perf --model llama-50m --layout packed --optimizer-layout zero1
+    python -m maltos_amd.train_perf --model llama-50m --layout dense  --graph
     python -m maltos_amd.train_perf --model llama-tiny --shards tests/golden/tokens_0000*.bin --seq-len 31
 
 What it does is what the reference's `tools/profile_train_perf.py` does around its timed region (:470-548 synthetic
@@ -79,7 +80,7 @@ def make_synthetic_batch(*, batch_size: int, seq_len: int, vocab_size: int, layo
 
 def run(args: argparse.Namespace) -> dict:
     from .grad_clip import clip_grad_norm_
-    from .llama import LlamaConfig, LlamaForCausalLM
+    from .llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
     from .optim import FusedAdamW, MasterWeightsOptimizer
     from .zero1 import Zero1FlatBuffers
 
@@ -95,6 +96,7 @@ def run(args: argparse.Namespace) -> dict:
             if p.dim() >= 2:
                 p.normal_(0.0, 0.02)
     model = model.to(dev).to(dtype)
+    set_grad_accumulation_into_buffers(model)   # weight gradients add into bound gradient buffers where there are any
     adamw = lambda ps: FusedAdamW(ps, lr=args.lr, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
     factory = (lambda ps: MasterWeightsOptimizer(ps, optimizer_factory=adamw)) if dtype == torch.bfloat16 else adamw
     zero = Zero1FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=args.bucket_mb) if args.optimizer_layout == "zero1" else None
@@ -112,13 +114,23 @@ def run(args: argparse.Namespace) -> dict:
         source = {"synthetic": args.layout}
 
     losses, norms, times = [], [], []
+    captured = None
+    if args.graph:
+        from .graph_step import CapturedForwardBackward
+        if zero:
+            zero.reset_grads()
+        clear = zero.reset_grads if zero else (lambda: opt.zero_grad(set_to_none=True))
+        captured = CapturedForwardBackward(model, next_batch(), embed=model.embed_tokens, clear_grads=clear)
 
     def step() -> None:
         batch = next_batch()
         if zero:
             zero.reset_grads()
-        loss = model(batch)
-        loss.backward()
+        if captured is not None:
+            loss = captured(batch).clone()
+        else:
+            loss = model(batch)
+            loss.backward()
         if zero:
             norm = zero.step(args.max_grad_norm)
         else:
@@ -141,7 +153,7 @@ def run(args: argparse.Namespace) -> dict:
     mean = sum(times) / len(times)
     return {
         "model": args.model, "dtype": args.dtype, "batch_size": args.batch_size, "seq_len": args.seq_len, "data": source,
-        "optimizer_layout": args.optimizer_layout, "buckets": len(zero.buckets) if zero else None,
+        "optimizer_layout": args.optimizer_layout, "graph": bool(args.graph), "buckets": len(zero.buckets) if zero else None,
         "params": sum(p.numel() for p in model.parameters()), "steps": args.steps, "warmup": args.warmup,
         "step_ms_mean": mean * 1e3, "step_ms_median": statistics.median(times) * 1e3, "step_ms_min": min(times) * 1e3,
         "tokens_per_sec": tokens / mean, "model_tflops": tokens * model.flops_per_token() / mean / 1e12,
@@ -155,6 +167,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--layout", choices=["dense", "packed"], default="dense")
     ap.add_argument("--optimizer-layout", choices=["flat", "zero1"], default="flat")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay forward + backward from one HIP graph (bf16, fixed batch shapes; see maltos_amd.graph_step)")
     ap.add_argument("--bucket-mb", type=int, default=25)
     ap.add_argument("--shards", nargs="*", default=[], help="token shard files (raw little-endian uint32) instead of synthetic ids")
     ap.add_argument("--batch-size", type=int, default=8)

@@ -41,8 +41,9 @@ def test_synthetic_batches_are_valid_causal_lm_batches(layout):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("extra", [["--layout", "dense"], ["--layout", "packed", "--optimizer-layout", "zero1"],
-                                   ["--shards", "tests/golden/tokens_0000*.bin", "--seq-len", "31", "--batch-size", "4"]],
-                         ids=["dense", "packed-zero1", "shards"])
+                                   ["--shards", "tests/golden/tokens_0000*.bin", "--seq-len", "31", "--batch-size", "4"],
+                                   ["--layout", "packed", "--graph"], ["--layout", "dense", "--graph", "--optimizer-layout", "zero1"]],
+                         ids=["dense", "packed-zero1", "shards", "packed-graph", "dense-graph-zero1"])
 def test_runner_steps_and_reports(dev, tmp_path, extra):
     out = tmp_path / "summary.json"
     argv = ["--model", "llama-tiny", "--batch-size", "2", "--seq-len", "256", "--steps", "3", "--warmup", "1", "--out", str(out), *extra]
@@ -52,3 +53,10 @@ def test_runner_steps_and_reports(dev, tmp_path, extra):
     assert 0 < s["loss_last"] < 12 and s["grad_norm_last"] > 0
     if "zero1" in extra:
         assert s["buckets"] >= 1
+    assert s["graph"] == ("--graph" in extra)
+    if "--graph" in extra:      # the same run without the graph gives the same loss (the steps are deterministic)
+        eager = tmp_path / "eager.json"
+        assert tp.main([a for a in argv if a != "--graph"] + ["--out", str(eager)]) == 0   # the later --out wins
+        e = json.loads(eager.read_text())
+        assert abs(e["loss_last"] - s["loss_last"]) <= 1e-6 * abs(e["loss_last"])
+        assert abs(e["grad_norm_last"] - s["grad_norm_last"]) <= 1e-5 * abs(e["grad_norm_last"])
