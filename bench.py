@@ -154,6 +154,64 @@ def bench_adamw(torch, ops, _lib, dev, steps, warmup):
             "frac_of_hbm_peak": bytes_per_launch / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
 
+def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
+    """The memory-bound kernels of the step, each alone at its LLaMA-50M shape (merge: at the ring configuration's), timed
+    with the library's HIP events: microseconds per call, algorithmic bytes (every operand read once, every result
+    written once), GB/s and the fraction of the HBM peak."""
+    N, h, I, V = 8 * 2048, 512, 1376, 32000
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(1234)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).to(bf).to(dev)
+    x, res, dy, dres = rnd(N, h), rnd(N, h), rnd(N, h), rnd(N, h)
+    w = torch.ones(h, dtype=bf, device=dev)
+    _, rstd = torch.ops.maltos.rmsnorm_fwd(x, w, 1e-5)
+    gate, up, dh = rnd(N, I), rnd(N, I), rnd(N, I)
+    q = rnd(8, 2048, 8, 64).transpose(1, 2)                      # the projection output's [B, H, S, D] view
+    ang = torch.arange(2048, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(0, 64, 2, dtype=torch.float32) / 64))[None, :]
+    cos, sin = torch.cos(ang).to(bf).to(dev), torch.sin(ang).to(bf).to(dev)
+    logits = rnd(N, V)
+    labels = torch.randint(0, V, (N,), generator=g).to(dev)
+    n_par = 58_073_600
+    gsrc = torch.randn(n_par, device=dev).to(bf)
+    gdst = torch.empty(n_par, device=dev)
+    sq = torch.empty((), dtype=torch.float64, device=dev)
+    B4, H4, S4, D4 = 1, 16, 8192, 128
+    out_acc = torch.zeros(B4, H4, S4, D4, device=dev)
+    lse_acc = torch.zeros(B4, H4, S4, device=dev)
+    o_blk = torch.randn(B4, H4, S4, D4, device=dev).to(bf)
+    lse_blk = torch.randn(B4, H4, S4, device=dev)
+    e = 2
+    cases = [
+        ("rmsnorm_fwd", "rmsnorm_fwd", 2 * N * h * e, lambda: torch.ops.maltos.rmsnorm_fwd(x, w, 1e-5)),
+        ("rmsnorm_bwd", "rmsnorm_bwd", 3 * N * h * e, lambda: torch.ops.maltos.rmsnorm_bwd(dy, x, w, rstd)),
+        ("add_rmsnorm_fwd", "rmsnorm_fwd", 4 * N * h * e, lambda: torch.ops.maltos.add_rmsnorm_fwd(x, res, w, 1e-5)),
+        ("add_rmsnorm_bwd", "rmsnorm_bwd", 4 * N * h * e, lambda: torch.ops.maltos.add_rmsnorm_bwd(dy, dres, x, w, rstd)),
+        ("rope", "rope", 2 * e * q.numel(), lambda: ops.rope(q, cos, sin)),
+        ("swiglu_fwd", "swiglu_fwd", 3 * N * I * e, lambda: torch.ops.maltos.swiglu_fwd(gate, up)),
+        ("swiglu_bwd", "swiglu_bwd", 5 * N * I * e, lambda: torch.ops.maltos.swiglu_bwd(dh, gate, up)),
+        ("cross_entropy_fwd_bwd", "ce", 2 * N * V * e, lambda: torch.ops.maltos.ce_fwd_bwd(logits, labels, -100)),
+        ("grad_to_f32_with_norm", "grad_to_f32", 6 * n_par, lambda: ops.grad_to_f32_(gdst, gsrc, sq_out=sq)),
+        ("attn_merge", "attn_merge", 10 * B4 * H4 * S4 * D4 + 12 * B4 * H4 * S4,
+         lambda: ops.attention_merge_(out_acc, lse_acc, o_blk, lse_blk)),
+    ]
+    out = {}
+    with torch.no_grad():
+        for label, timer, nbytes, fn in cases:
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            _lib.kernel_timing(True)
+            for _ in range(reps):
+                fn()
+            torch.cuda.synchronize()
+            total_ms, launches = _lib.kernel_time_ms(timer)
+            _lib.kernel_timing(False)
+            us = total_ms / max(1, launches) * 1e3
+            gbps = nbytes / (us * 1e-6) / 1e9
+            out[label] = {"us": us, "algorithmic_bytes": nbytes, "gbps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
+    return out
+
+
 def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False):
     """graph=True: forward + backward replayed from one HIP graph (clip, AdamW and the gradient clear stay eager).
     zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
@@ -302,6 +360,7 @@ def main() -> int:
         if "attn_bwd_dq_ds" in kernels:
             extra["attn_recompute_backward"] = bench_attention_recompute(args)
         extra["adamw_flat_fp32"] = bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup)
+        extra["hbm_kernels"] = bench_hbm_kernels(torch, ops, _lib, dev)
         extra["llama50m_train_step"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup))
         extra["llama50m_train_step_graph"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup), graph=True)
         extra["llama50m_train_step_zero1_layout"] = bench_llama50m(torch, dev, max(5, args.steps // 2), max(10, args.warmup),

@@ -233,6 +233,7 @@ extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk
   MLTS_REQUIRE(out_acc && lse_acc && o_blk && lse_blk && o_blk_stride, "mlts_attn_merge: null pointer");
   MLTS_REQUIRE((D & 3) != 0 || mlts_aligned16(out_acc), "mlts_attn_merge: out_acc must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  MltsKernelTimer timer("attn_merge", st);
   const int64_t total_rows = static_cast<int64_t>(B) * H * q_len;
   int G = 1;
   while (G < (D + 3) / 4 && G < 64) G <<= 1;

@@ -399,6 +399,7 @@ int rmsnorm_bwd_t(const void* dy, const void* x, const void* w, const float* rst
 template <typename T>
 int rope_t(const void* x, const int64_t* xs, void* y, const int64_t* ys, const void* ct, const void* sn, int max_pos,
            const int32_t* positions, int off, int B, int H, int S, int D, int inverse, hipStream_t st) {
+  MltsKernelTimer timer("rope", st);
   constexpr int N = Vec16<T>::N;
   const int64_t total = static_cast<int64_t>(B) * S * H * (D / N);
   const int64_t blocks = (total + kThreads - 1) / kThreads;
@@ -416,6 +417,7 @@ int rope_t(const void* x, const int64_t* xs, void* y, const int64_t* ys, const v
 
 template <typename T>
 int swiglu_fwd_t(const void* g, const void* u, void* h, int64_t n, bool vec, hipStream_t st) {
+  MltsKernelTimer timer("swiglu_fwd", st);
   constexpr int N = Vec16<T>::N;
   int64_t done = 0;
   if (vec && n >= N) {
@@ -435,6 +437,7 @@ int swiglu_fwd_t(const void* g, const void* u, void* h, int64_t n, bool vec, hip
 template <typename T>
 int swiglu_bwd_t(const void* dh, const void* g, const void* u, void* dg, void* du, int64_t n, bool vec,
                  hipStream_t st) {
+  MltsKernelTimer timer("swiglu_bwd", st);
   constexpr int N = Vec16<T>::N;
   int64_t done = 0;
   if (vec && n >= N) {

@@ -144,6 +144,85 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* __restrict_
   }
 }
 
+// Row kept in registers: NV 16-byte vectors per lane (a 32000-entry bf16 row is 8 per lane of a 512-lane block), all
+// loads of a row issued before the first use.  No LDS beyond the reduction scratch, so four or more rows are in
+// flight per CU instead of the two that fit when rows are staged in LDS.
+template <typename T, int NV>
+__global__ __launch_bounds__(kCeThreads) void ce_row_reg_kernel(const T* __restrict__ logits,
+                                                                const int64_t* __restrict__ labels, T* __restrict__ dlogits,
+                                                                float* __restrict__ row_loss,
+                                                                const int32_t* __restrict__ count, int vocab,
+                                                                int64_t ignore_index) {
+  constexpr int N = Vec16<T>::N;
+  __shared__ float red[kCeWaves];
+  const int64_t row = blockIdx.x;
+  const int64_t label = labels[row];
+  const T* zr = logits + row * vocab;
+  T* dr = dlogits + row * vocab;
+  const int nvec = vocab / N;
+  if (label == ignore_index) {
+    if (threadIdx.x == 0) row_loss[row] = 0.f;
+    Vec16<T> z;
+#pragma unroll
+    for (int j = 0; j < N; ++j) z.set(j, 0.f);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = threadIdx.x + i * kCeThreads;
+      if (c < nvec) __builtin_nontemporal_store(z.v, reinterpret_cast<decltype(z.v)*>(dr) + c);
+    }
+    return;
+  }
+  const bool label_ok = label >= 0 && label < vocab;
+  Vec16<T> t[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kCeThreads;
+    if (c < nvec) t[i].v = __builtin_nontemporal_load(reinterpret_cast<const decltype(t[i].v)*>(zr) + c);
+  }
+  float label_logit = 0.f;
+  if (threadIdx.x == 0 && label_ok) label_logit = to_f32<T>(zr[label]);
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (threadIdx.x + i * kCeThreads < nvec) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) mx = fmaxf(mx, t[i].get(j));
+    }
+  }
+  mx = block_max(mx, red);
+  const float mxs = mx * kLog2e;
+  float se = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (threadIdx.x + i * kCeThreads < nvec) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) se += exp2f(t[i].get(j) * kLog2e - mxs);
+    }
+  }
+  se = block_sum(se, red);
+  const float lse = mx + logf(se);
+  if (threadIdx.x == 0) row_loss[row] = label_ok ? lse - label_logit : NAN;
+  const int cnt = *count;
+  const float inv = 1.0f / static_cast<float>(cnt > 0 ? cnt : 1);
+  const float lses = lse * kLog2e;
+  const int lvec = label_ok ? static_cast<int>(label / N) : -1;
+  const int lsub = label_ok ? static_cast<int>(label % N) : 0;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * kCeThreads;
+    if (c < nvec) {
+      Vec16<T> o;
+#pragma unroll
+      for (int j = 0; j < N; ++j) {
+        float p = exp2f(t[i].get(j) * kLog2e - lses);
+        if (c == lvec && j == lsub) p -= 1.0f;
+        o.set(j, p * inv);
+      }
+      __builtin_nontemporal_store(o.v, reinterpret_cast<decltype(o.v)*>(dr) + c);
+    }
+  }
+}
+
 __global__ __launch_bounds__(kCeThreads) void ce_loss_reduce_kernel(const float* __restrict__ row_loss, int64_t rows,
                                                                     const int32_t* __restrict__ count,
                                                                     float* __restrict__ loss_out) {
@@ -200,6 +279,18 @@ int ce_launch(const void* logits, const int64_t* labels, void* dlogits, float* r
   const size_t smem = staged ? static_cast<size_t>((row_bytes + 15) & ~15LL) : 0;
   const T* lg = static_cast<const T*>(logits);
   T* dl = static_cast<T*>(dlogits);
+  if (vec && vocab / N <= 8 * kCeThreads) {  // the row fits the registers of one block
+    const int per_lane = (vocab / N + kCeThreads - 1) / kCeThreads;
+#define MLTS_CE_REG(NV)                                                                                              \
+  hipLaunchKernelGGL((ce_row_reg_kernel<T, NV>), dim3((unsigned)rows), dim3(kCeThreads), 0, st, lg, labels, dl, row_loss, \
+                     count, vocab, ignore_index)
+    if (per_lane <= 1) MLTS_CE_REG(1);
+    else if (per_lane <= 2) MLTS_CE_REG(2);
+    else if (per_lane <= 4) MLTS_CE_REG(4);
+    else MLTS_CE_REG(8);
+#undef MLTS_CE_REG
+    return MLTS_OK;
+  }
 #define MLTS_CE_LAUNCH(ST, VC)                                                                                      \
   do {                                                                                                              \
     auto kern = ce_row_kernel<T, ST, VC>;                                                                           \
