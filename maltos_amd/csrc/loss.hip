@@ -146,9 +146,10 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* __restrict_
 
 // Row kept in registers: NV 16-byte vectors per lane (a 32000-entry bf16 row is 8 per lane of a 512-lane block), all
 // loads of a row issued before the first use.  No LDS beyond the reduction scratch, so four or more rows are in
-// flight per CU instead of the two that fit when rows are staged in LDS.
+// flight per CU instead of the two that fit when rows are staged in LDS (six wavefronts per SIMD = three blocks per CU
+// is the register budget that still compiles without spills for eight vectors per lane).
 template <typename T, int NV>
-__global__ __launch_bounds__(kCeThreads) void ce_row_reg_kernel(const T* __restrict__ logits,
+__global__ __launch_bounds__(kCeThreads, 6) void ce_row_reg_kernel(const T* __restrict__ logits,
                                                                 const int64_t* __restrict__ labels, T* __restrict__ dlogits,
                                                                 float* __restrict__ row_loss,
                                                                 const int32_t* __restrict__ count, int vocab,
