@@ -216,7 +216,9 @@ int rmsnorm_bwd_blocks(int64_t rows) {
 
 // ============================== RoPE =====================================================
 // One lane rotates the pairs inside one 16-byte vector of a [b, h, s, :] row.
-template <typename T, bool INVERSE>
+// IDX is the type the flat element index is taken apart in: 32-bit whenever the tensor has fewer than 2^31 vectors
+// (three 64-bit divisions per lane cost several hundred instructions, more than the rotation itself).
+template <typename T, bool INVERSE, typename IDX>
 __global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
                                                         T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
                                                         const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
@@ -225,27 +227,30 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x,
   constexpr int N = Vec16<T>::N;
   const int vec_per_row = D / N;
   const int64_t total = static_cast<int64_t>(B) * S * H * vec_per_row;
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  if (idx >= total) return;
+  const int64_t idx64 = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (idx64 >= total) return;
   // order (b, s, h, vec): neighbouring lanes touch neighbouring memory for [B, S, H, D] storage
-  const int vc = static_cast<int>(idx % vec_per_row);
-  int64_t rest = idx / vec_per_row;
-  const int h = static_cast<int>(rest % H);
-  rest /= H;
-  const int s = static_cast<int>(rest % S);
-  const int b = static_cast<int>(rest / S);
+  const IDX idx = static_cast<IDX>(idx64);
+  const int vc = static_cast<int>(idx % static_cast<IDX>(vec_per_row));
+  IDX rest = idx / static_cast<IDX>(vec_per_row);
+  const int h = static_cast<int>(rest % static_cast<IDX>(H));
+  rest /= static_cast<IDX>(H);
+  const int s = static_cast<int>(rest % static_cast<IDX>(S));
+  const int b = static_cast<int>(rest / static_cast<IDX>(S));
   int pos = positions ? positions[static_cast<int64_t>(b) * S + s] : position_offset + s;
   pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);  // host validated; keeps reads in bounds
   const T* xp = x + b * xsb + h * xsh + s * xss + vc * N;
   T* yp = y + b * ysb + h * ysh + s * yss + vc * N;
   Vec16<T> xv = *reinterpret_cast<const Vec16<T>*>(xp);
-  const T* cp = cos_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2);
-  const T* sp = sin_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2);
+  // the N / 2 table entries of this vector are 8 bytes (4 bf16 or 2 fp32), 8-byte aligned: one load each
+  struct alignas(8) Half8 { T v[N / 2]; };
+  const Half8 cv = *reinterpret_cast<const Half8*>(cos_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2));
+  const Half8 sv = *reinterpret_cast<const Half8*>(sin_tab + static_cast<int64_t>(pos) * (D / 2) + vc * (N / 2));
   Vec16<T> o;
 #pragma unroll
   for (int j = 0; j < N / 2; ++j) {
-    const float c = to_f32<T>(cp[j]);
-    float sn = to_f32<T>(sp[j]);
+    const float c = to_f32<T>(cv.v[j]);
+    float sn = to_f32<T>(sv.v[j]);
     const float xe = xv.get(2 * j), xo = xv.get(2 * j + 1);
     float oe, oo;
     if (!INVERSE) {
@@ -404,14 +409,19 @@ int rope_t(const void* x, const int64_t* xs, void* y, const int64_t* ys, const v
   const int64_t total = static_cast<int64_t>(B) * S * H * (D / N);
   const int64_t blocks = (total + kThreads - 1) / kThreads;
   if (blocks == 0) return MLTS_OK;
-  if (inverse)
-    hipLaunchKernelGGL((rope_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
-                       xs[0], xs[1], xs[2], static_cast<T*>(y), ys[0], ys[1], ys[2], static_cast<const T*>(ct),
-                       static_cast<const T*>(sn), max_pos, positions, off, B, H, S, D);
-  else
-    hipLaunchKernelGGL((rope_kernel<T, false>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x),
-                       xs[0], xs[1], xs[2], static_cast<T*>(y), ys[0], ys[1], ys[2], static_cast<const T*>(ct),
-                       static_cast<const T*>(sn), max_pos, positions, off, B, H, S, D);
+#define MLTS_ROPE(INV, IDX)                                                                                         \
+  hipLaunchKernelGGL((rope_kernel<T, INV, IDX>), dim3((unsigned)blocks), dim3(kThreads), 0, st, static_cast<const T*>(x), \
+                     xs[0], xs[1], xs[2], static_cast<T*>(y), ys[0], ys[1], ys[2], static_cast<const T*>(ct),         \
+                     static_cast<const T*>(sn), max_pos, positions, off, B, H, S, D)
+  const bool narrow = total < (1LL << 31);
+  if (inverse) {
+    if (narrow) MLTS_ROPE(true, uint32_t);
+    else MLTS_ROPE(true, int64_t);
+  } else {
+    if (narrow) MLTS_ROPE(false, uint32_t);
+    else MLTS_ROPE(false, int64_t);
+  }
+#undef MLTS_ROPE
   return mlts_check_launch("mlts_rope");
 }
 
@@ -548,6 +558,8 @@ extern "C" int mlts_rope(const void* x, const int64_t x_stride[3], void* y, cons
   MLTS_REQUIRE(positions != nullptr || (position_offset >= 0 && position_offset + S <= max_pos),
                "mlts_rope: positions [%d, %d) exceed the table (%d rows)", position_offset, position_offset + S, max_pos);
   MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(y), "mlts_rope: x and y must be 16-byte aligned");
+  MLTS_REQUIRE((reinterpret_cast<uintptr_t>(cos_tab) & 7u) == 0 && (reinterpret_cast<uintptr_t>(sin_tab) & 7u) == 0,
+               "mlts_rope: the cos / sin tables must be 8-byte aligned");
   for (int i = 0; i < 3; ++i)
     MLTS_REQUIRE((x_stride[i] * esz) % 16 == 0 && (y_stride[i] * esz) % 16 == 0,
                  "mlts_rope: strides must keep rows 16-byte aligned");
