@@ -344,6 +344,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     // masked tiles only (a wave-uniform branch around VALU work, no matrix instruction inside): hidden scores -> -inf
     auto apply_mask = [&](auto qb_tag, f32x16& s) {
       constexpr int qb = decltype(qb_tag)::value;
+      // the comparisons below belong to masked tiles only: an opaque copy of their operand keeps the compiler from
+      // hoisting all of them in front of the wave-uniform branch, where every tile would pay for them
+      int causal_here = causal_t;
+      asm volatile("" : "+v"(causal_here));
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int qrow = qb * 32 + g * 8 + hh * 4;
@@ -361,7 +365,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         for (int r = 0; r < 4; ++r) {
           bool vis;
           if (MODE == MLTS_MASK_CAUSAL) {
-            vis = causal_t <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
+            vis = causal_here <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
           } else {
             const int qi = q0 + qrow + r;
             vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
