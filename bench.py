@@ -93,6 +93,7 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup):
         total_ms, launches = _lib.kernel_time_ms(name)
         if launches:
             kernels[name] = {"ms": total_ms / launches, "launches_per_step": launches / steps}
+    delta_time = _lib.kernel_time_ms("attn_delta")
     _lib.kernel_timing(False)
     # algorithmic flops per launch of each kernel (FlashAttention convention: 2 GEMMs forward, 5 backward: S, dP, dV,
     # dK, dQ, each fwd_flops / 2)
@@ -107,6 +108,12 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup):
         kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops
     for name, rec in kernels.items():
         rec["tflops"] = kernel_flops[name] / (rec["ms"] * 1e-3) / 1e12
+    # the row-wise delta = sum(dO * O) pass in front of the backward kernels: memory bound, reads dO and O once
+    total_ms, launches = delta_time
+    if launches:
+        nbytes = 2 * 2 * B * H * S * D + 4 * B * H * S
+        kernels["attn_delta"] = {"ms": total_ms / launches, "launches_per_step": launches / steps,
+                                 "gbps": nbytes / (total_ms / launches * 1e-3) / 1e9}
     return sec, flops, kernels, kernel_flops
 
 
@@ -194,6 +201,7 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
         ("attn_merge", "attn_merge", 10 * B4 * H4 * S4 * D4 + 12 * B4 * H4 * S4,
          lambda: ops.attention_merge_(out_acc, lse_acc, o_blk, lse_blk)),
     ]
+
     out = {}
     with torch.no_grad():
         for label, timer, nbytes, fn in cases:

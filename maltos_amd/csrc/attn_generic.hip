@@ -319,7 +319,8 @@ __global__ __launch_bounds__(GT) void attn_delta_kernel(const T* __restrict__ do
 
 // bf16, head_dim a multiple of 8, 16-byte aligned rows: D / 8 lanes share a row (one 16-byte load of dO and of O per
 // lane), four rows per lane group in flight.  The plain kernel above reads two bytes per lane and reaches 3 TB/s.
-template <int LPR>  // lanes per row, a power of two <= 32
+// IDX: type the row index is split in (32-bit below 2^31 rows: 64-bit divisions would dominate the kernel).
+template <int LPR, typename IDX>  // lanes per row, a power of two <= 32
 __global__ __launch_bounds__(256) void attn_delta_vec_kernel(const bf16_t* __restrict__ dout, int64_t ds0, int64_t ds1, int64_t ds2,
                                                               const bf16_t* __restrict__ o, int64_t os0, int64_t os1, int64_t os2,
                                                               float* __restrict__ delta, int H, int S, int64_t total, int D) {
@@ -331,10 +332,11 @@ __global__ __launch_bounds__(256) void attn_delta_vec_kernel(const bf16_t* __res
   v4i32 a[UNROLL], c[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const int64_t row = min(row0 + u * RPB, total - 1);
-    const int s = static_cast<int>(row % S);
-    const int h = static_cast<int>((row / S) % H);
-    const int64_t b = row / (static_cast<int64_t>(S) * H);
+    const IDX row = static_cast<IDX>(min(row0 + u * RPB, total - 1));
+    const IDX bh = row / static_cast<IDX>(S);
+    const int s = static_cast<int>(row - bh * static_cast<IDX>(S));
+    const int64_t b = static_cast<int64_t>(bh / static_cast<IDX>(H));
+    const int h = static_cast<int>(bh - static_cast<IDX>(b) * static_cast<IDX>(H));
     a[u] = v4i32{0, 0, 0, 0};
     c[u] = v4i32{0, 0, 0, 0};
     if (sub * 8 < D) {
@@ -434,6 +436,7 @@ int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const i
                     int S, int D, int dtype, hipStream_t st) {
   const int64_t rows = static_cast<int64_t>(B) * H * S;
   if (rows == 0) return MLTS_OK;
+  MltsKernelTimer timer("attn_delta", st);
   const bool vec = dtype == MLTS_BF16 && D % 8 == 0 && D <= 256 && ((dos[0] | dos[1] | dos[2] | os[0] | os[1] | os[2]) & 7) == 0 &&
                    mlts_aligned16(dout) && mlts_aligned16(o);
   if (vec) {
@@ -442,12 +445,18 @@ int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const i
     const unsigned nb = static_cast<unsigned>((rows + rows_per_block - 1) / rows_per_block);
     const bf16_t* dp = static_cast<const bf16_t*>(dout);
     const bf16_t* op = static_cast<const bf16_t*>(o);
-#define MLTS_DELTA(LPR) \
-  hipLaunchKernelGGL(attn_delta_vec_kernel<LPR>, dim3(nb), dim3(256), 0, st, dp, dos[0], dos[1], dos[2], op, os[0], os[1], os[2], delta, H, S, rows, D)
+#define MLTS_DELTA_IDX(LPR, IDX) \
+  hipLaunchKernelGGL((attn_delta_vec_kernel<LPR, IDX>), dim3(nb), dim3(256), 0, st, dp, dos[0], dos[1], dos[2], op, os[0], os[1], os[2], delta, H, S, rows, D)
+#define MLTS_DELTA(LPR)                                  \
+  do {                                                   \
+    if (rows < (1LL << 31)) MLTS_DELTA_IDX(LPR, uint32_t); \
+    else MLTS_DELTA_IDX(LPR, int64_t);                   \
+  } while (0)
     if (lpr == 8) MLTS_DELTA(8);
     else if (lpr == 16) MLTS_DELTA(16);
     else MLTS_DELTA(32);
 #undef MLTS_DELTA
+#undef MLTS_DELTA_IDX
     return mlts_check_launch("mlts_attn_delta");
   }
   const int64_t blocks = (rows + (GT / 64) - 1) / (GT / 64);
