@@ -100,15 +100,27 @@ template <typename T>
 __global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc, float* __restrict__ lse_acc,
                                                     const T* __restrict__ o_blk, int64_t bs0, int64_t bs1, int64_t bs2,
                                                     const float* __restrict__ lse_blk, int H, int S, int D, int q_off,
-                                                    int q_len, int64_t total_rows, int G) {
+                                                    int q_len, int64_t total_rows, int G, int blk_vec) {
   const int vec_per_row = D >> 2;
   const int rows_per_block = 256 / G;
   const int64_t rowi = static_cast<int64_t>(blockIdx.x) * rows_per_block + threadIdx.x / G;
   const int sub = threadIdx.x % G;
   if (rowi >= total_rows) return;
-  const int i = static_cast<int>(rowi % q_len);
-  const int64_t bh = rowi / q_len;
-  const int h = static_cast<int>(bh % H), b = static_cast<int>(bh / H);
+  // 32-bit divisions whenever they suffice (a wave-uniform choice): three 64-bit ones cost more than the merge itself
+  int i, h, b;
+  int64_t bh;
+  if (total_rows < (1LL << 31)) {
+    const uint32_t r = static_cast<uint32_t>(rowi), bh32 = r / static_cast<uint32_t>(q_len);
+    i = static_cast<int>(r - bh32 * static_cast<uint32_t>(q_len));
+    b = static_cast<int>(bh32 / static_cast<uint32_t>(H));
+    h = static_cast<int>(bh32 - static_cast<uint32_t>(b) * static_cast<uint32_t>(H));
+    bh = bh32;
+  } else {
+    i = static_cast<int>(rowi % q_len);
+    bh = rowi / q_len;
+    h = static_cast<int>(bh % H);
+    b = static_cast<int>(bh / H);
+  }
   const int64_t arow = bh * S + q_off + i;
   const float la = lse_acc[arow], lb = lse_blk[bh * q_len + i];
   const float mx = fmaxf(la, lb);
@@ -122,9 +134,17 @@ __global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc,
   if ((D & 3) == 0) {
     for (int vc = sub; vc < vec_per_row; vc += G) {
       const f32x4 acc = reinterpret_cast<const f32x4*>(out_acc + arow * D)[vc];
+      struct alignas(4 * sizeof(T)) Blk4 { T v[4]; };   // one 8- or 16-byte load where the block's layout allows it
+      Blk4 blk4;
+      if (blk_vec) {
+        blk4 = *reinterpret_cast<const Blk4*>(bp + vc * 4);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) blk4.v[e] = bp[vc * 4 + e];
+      }
       f32x4 r;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[e] = acc[e] * pa + to_f32<T>(bp[vc * 4 + e]) * pb;
+      for (int e = 0; e < 4; ++e) r[e] = acc[e] * pa + to_f32<T>(blk4.v[e]) * pb;
       reinterpret_cast<f32x4*>(out_acc + arow * D)[vc] = r;
     }
   } else {
@@ -239,13 +259,16 @@ extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk
   while (G < (D + 3) / 4 && G < 64) G <<= 1;
   const int rows_per_block = 256 / G;
   const int64_t blocks = (total_rows + rows_per_block - 1) / rows_per_block;
+  const uintptr_t blk_bytes4 = blk_dtype == MLTS_BF16 ? 8 : 16;  // four elements of the block
+  const int blk_vec = (reinterpret_cast<uintptr_t>(o_blk) % blk_bytes4 == 0) &&
+                      ((o_blk_stride[0] | o_blk_stride[1] | o_blk_stride[2]) & 3) == 0;
   if (blk_dtype == MLTS_BF16)
     hipLaunchKernelGGL(merge_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, out_acc, lse_acc,
                        static_cast<const bf16_t*>(o_blk), o_blk_stride[0], o_blk_stride[1], o_blk_stride[2], lse_blk, H, S,
-                       D, q_off, q_len, total_rows, G);
+                       D, q_off, q_len, total_rows, G, blk_vec);
   else
     hipLaunchKernelGGL(merge_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, st, out_acc, lse_acc,
                        static_cast<const float*>(o_blk), o_blk_stride[0], o_blk_stride[1], o_blk_stride[2], lse_blk, H, S,
-                       D, q_off, q_len, total_rows, G);
+                       D, q_off, q_len, total_rows, G, blk_vec);
   return mlts_check_launch("mlts_attn_merge");
 }
