@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
 # by the same counters over the --calibrate-traffic kernel (summary: profiles/attn_cfg2_hbm_traffic.md).  Counters
 # cannot be read from inside the timed run, so the figures are carried here and refreshed with the profile.
 MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 679.1e6, "attn_bwd_dkdv": 1965.8e6, "attn_bwd_dq_ds": 1425.9e6,
-                              # the recomputing dQ kernel and the dK/dV kernel without the dS hand-over (MLTS_BWD_DS_MAX_MB=0)
+                              # the recomputing dQ kernel and the dK/dV kernel without the dS hand-over (the default backward)
                               "attn_bwd_dq": 651.3e6, "attn_bwd_dkdv_recompute": 885.8e6}
 
 
@@ -117,19 +117,17 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup):
     return sec, flops, kernels, kernel_flops
 
 
-def bench_attention_recompute(args):
-    """The same attention step with MLTS_BWD_DS_MAX_MB=0: the dQ kernel recomputes S and dP instead of reading dS from
-    the dK/dV kernel (workspace O(S) instead of 2 bytes per score).  The choice is read once per process, so this
-    runs in a child process."""
-    import subprocess
-    cmd = [sys.executable, os.path.abspath(__file__), "--skip-extra", "--skip-cpu", "--steps", str(args.steps),
-           "--warmup", str(args.warmup)]
-    proc = subprocess.run(cmd, env={**os.environ, "MLTS_BWD_DS_MAX_MB": "0"}, capture_output=True, text=True, timeout=600)
-    if proc.returncode != 0:
-        raise RuntimeError(f"recompute-backward leg failed:\n{proc.stderr[-2000:]}")
-    r = json.loads(proc.stdout.strip().splitlines()[-1])
-    return {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "kernels": r["kernels"],
-            "workspace": "lse2 + delta + tile statistics only"}
+def bench_attention_handover(torch, ops, _lib, dev, steps, warmup):
+    """The same attention step with the dS hand-over allowed (ops.set_backward_ds_handover_limit): the dK/dV kernel
+    stores dS (2 bytes per score, 2.1 GB of workspace at this shape) and the dQ kernel reads it instead of recomputing
+    S and dP.  The default backward recomputes and keeps the workspace O(B * H * S)."""
+    previous = ops.set_backward_ds_handover_limit(4 << 30)
+    try:
+        sec, flops, kernels, _ = bench_attention(torch, ops, _lib, dev, steps, warmup)
+    finally:
+        ops.set_backward_ds_handover_limit(previous)
+    return {"value": (flops["fwd"] + flops["bwd"]) / sec / 1e12, "unit": "TFLOP/s", "ms_per_step": sec * 1e3,
+            "kernels": kernels, "workspace_bytes": 2 * 4 * 16 * 4096 * 4096}
 
 
 def bench_adamw(torch, ops, _lib, dev, steps, warmup):
@@ -375,8 +373,7 @@ def main() -> int:
                 torch.cuda.synchronize()
 
         half = max(5, args.steps // 2)
-        if "attn_bwd_dq_ds" in kernels:
-            leg("attn_recompute_backward", lambda: bench_attention_recompute(args))
+        leg("attn_ds_handover_backward", lambda: bench_attention_handover(torch, ops, _lib, dev, args.steps, args.warmup))
         leg("adamw_flat_fp32", lambda: bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup))
         leg("hbm_kernels", lambda: bench_hbm_kernels(torch, ops, _lib, dev))
         leg("llama50m_train_step", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup)))

@@ -81,9 +81,18 @@ typedef struct mlts_attn_shape {
  * (runtime/layers/flash_utils.py:105-135). */
 const char* mlts_attn_supports(const mlts_attn_shape* s);
 
-/* Bytes of device workspace mlts_attn_fwd / mlts_attn_bwd need for this shape. */
+/* Bytes of device workspace mlts_attn_fwd / mlts_attn_bwd need for this shape: the per-row statistics the kernels
+ * share (delta, LSE in base 2) and, with MLTS_MASK_DOC, the per-tile position / sequence-id ranges.  O(B * Hq * Sq),
+ * the workspace class of the flash backward the reference calls (runtime/layers/flash_utils.py:239-258). */
 int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s);
 int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32);
+
+/* Optional trade of memory for matrix work in mlts_attn_bwd: when the caller's workspace is at least
+ * mlts_attn_bwd_workspace_bytes + mlts_attn_bwd_ds_handover_bytes, the dK/dV kernel hands dS (bf16, 2 bytes per
+ * (query, key) pair: 2 * B * Hq * Sq * Sk bytes) to the dQ kernel instead of the dQ kernel recomputing the scores.
+ * Returns 0 for calls the hand-over does not serve (head_dim other than 128, MLTS_MASK_DOC, fp32 accumulation).
+ * With a smaller workspace the backward recomputes; results differ only in the rounding of dS. */
+int64_t mlts_attn_bwd_ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32);
 
 /* O = softmax(scale * Q K^T + mask) V and LSE = logsumexp (natural log, fp32, [B, Hq, Sq]).
  * Replaces F.scaled_dot_product_attention (utils/attention_backend.py:60-64,109-116),

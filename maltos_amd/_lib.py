@@ -67,6 +67,7 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_attn_supports": (C.c_char_p, [_SHAPE_P]),
     "mlts_attn_fwd_workspace_bytes": (C.c_int64, [_SHAPE_P]),
     "mlts_attn_bwd_workspace_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
+    "mlts_attn_bwd_ds_handover_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
     "mlts_attn_fwd": (C.c_int, [_SHAPE_P, _P, _P, _P, _P, _P, _P, C.c_int64, _P]),
     "mlts_attn_bwd": (
         C.c_int,

@@ -3,9 +3,12 @@
 // the log-sum-exp block merge.
 #include "attn_common.hpp"
 
-int mlts_attn_fwd_bf16(AttnParams p, int D, int mode, hipStream_t st);
-int mlts_attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);
-int64_t mlts_attn_bwd_bf16_workspace(const mlts_attn_shape* s, int accumulate_f32);
+int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st);                        // attn_fwd_dma.hip
+int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq);                             // attn_bwd_split.hip
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);    // attn_bwd_split.hip
+int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
+int64_t mlts_attn_bwd_ds_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t Sk);                              // attn_bwd_dq_ds.hip
+int mlts_attn_bwd_dq_bf16_ds(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_ds.hip
 int mlts_attn_generic_fwd(const AttnParams& p, int D, int dtype, int mode, hipStream_t st);
 int mlts_attn_generic_bwd(const AttnBwdParams& bp, int D, int dtype, int mode, hipStream_t st);
 int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const int64_t* os, float* delta, int B, int H,
@@ -14,7 +17,7 @@ int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const i
 namespace {
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~255LL; }
-inline int esize(int dtype) { return dtype == MLTS_BF16 ? 2 : 4; }
+constexpr int64_t kMaxRowStride = int64_t{1} << 24;  // the MFMA kernels address the rows of a tile with 32-bit element offsets
 
 bool uses_mfma(const mlts_attn_shape* s) { return s->dtype == MLTS_BF16 && (s->D == 64 || s->D == 128); }
 
@@ -38,6 +41,8 @@ const char* shape_problem(const mlts_attn_shape* s) {
     if (!strides_aligned(s->q_stride, 2) || !strides_aligned(s->k_stride, 2) || !strides_aligned(s->v_stride, 2) ||
         !strides_aligned(s->o_stride, 2))
       return "bf16 MFMA path needs strides that keep rows 16-byte aligned";
+    if (s->q_stride[2] >= kMaxRowStride || s->k_stride[2] >= kMaxRowStride || s->v_stride[2] >= kMaxRowStride)
+      return "bf16 MFMA path needs sequence strides below 2^24 elements";
   }
   return nullptr;
 }
@@ -153,59 +158,45 @@ __global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc,
   if (sub == 0) lse_acc[arow] = ln;
 }
 
-}  // namespace
 
-extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return shape_problem(s); }
-
-extern "C" int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s) {
-  if (shape_problem(s)) return -1;
-  return stats_bytes(s);
+// whether the dK/dV kernel may hand -dS to the dQ kernel for this call: head_dim 128 without a document mask and with
+// gradients in the input dtype (head_dim 64 has half the matrix work per pair and the same hand-over bytes, so
+// recomputing is faster there; gradients accumulated in fp32, the ring steps, keep the recomputed, once-rounded dS)
+int64_t ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32) {
+  if (!uses_mfma(s) || s->mask_mode == MLTS_MASK_DOC || s->D != 128 || accumulate_f32 || s->Sq == 0 || s->Sk == 0 || s->B == 0)
+    return 0;
+  return mlts_attn_bwd_ds_bytes(s->B, s->Hq, s->Sq, s->Sk);
 }
 
-extern "C" int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32) {
-  if (shape_problem(s)) return -1;
+int64_t bwd_min_workspace(const mlts_attn_shape* s) {
   const int64_t delta = align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
-  int64_t extra = 0;
-  if (uses_mfma(s)) extra = mlts_attn_bwd_bf16_workspace(s, accumulate_f32);
-  return stats_bytes(s) + delta + extra;
+  const int64_t lse2 = uses_mfma(s) ? mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq) : 0;
+  return stats_bytes(s) + delta + lse2;
 }
 
-extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o, float* lse,
-                             void* workspace, int64_t workspace_bytes, mlts_stream_t stream) {
-  const char* why = shape_problem(s);
-  MLTS_REQUIRE(why == nullptr, "mlts_attn_fwd: %s", why);
-  if (s->B == 0 || s->Sq == 0) return MLTS_OK;
-  MLTS_REQUIRE(q && o && lse, "mlts_attn_fwd: q, o, lse must be non-null");
-  MLTS_REQUIRE(s->Sk == 0 || (k && v), "mlts_attn_fwd: k, v must be non-null");
-  const int64_t need = stats_bytes(s);
-  MLTS_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), "mlts_attn_fwd: workspace too small (%lld < %lld)",
-               (long long)workspace_bytes, (long long)need);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  AttnParams p;
-  fill_params(p, s, q, k, v, o, lse);
-  if (uses_mfma(s)) {
-    MLTS_REQUIRE(mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) && mlts_aligned16(o),
-                 "mlts_attn_fwd: q, k, v, o must be 16-byte aligned");
-    setup_stats(p, s, static_cast<char*>(workspace), st);
-    return mlts_attn_fwd_bf16(p, s->D, s->mask_mode, st);
+// dK/dV kernel, then the dQ kernel: from the handed-over dS when ds_ws is set, by recomputation otherwise
+int attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* lse2_ws, void* ds_ws, hipStream_t st) {
+  const AttnParams& p = bp.a;
+  bp.nkt = (p.Sk + 127) / 128;
+  if (ds_ws) {
+    bp.ds_ws = ds_ws;
+    bp.ds_nkb = (p.Sk + 31) / 32;
+    bp.ds_nqt = (p.Sq + 63) / 64;
   }
-  return mlts_attn_generic_fwd(p, s->D, s->dtype, s->mask_mode, st);
+  int rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, lse2_ws, st);
+  if (rc != MLTS_OK) return rc;
+  return ds_ws ? mlts_attn_bwd_dq_bf16_ds(bp, D, mode, st) : mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
 }
 
-extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
-                             const void* k, const void* v, const void* o, const float* lse, void* dq,
-                             const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,
-                             const int64_t dv_stride[3], int accumulate_f32, void* workspace, int64_t workspace_bytes,
-                             mlts_stream_t stream) {
-  const char* why = shape_problem(s);
-  MLTS_REQUIRE(why == nullptr, "mlts_attn_bwd: %s", why);
-  if (s->B == 0 || (s->Sq == 0 && s->Sk == 0)) return MLTS_OK;
-  MLTS_REQUIRE(dout && q && k && v && o && lse && dq && dk && dv, "mlts_attn_bwd: null tensor pointer");
-  MLTS_REQUIRE(do_stride && dq_stride && dk_stride && dv_stride, "mlts_attn_bwd: null stride pointer");
-  const int64_t need = mlts_attn_bwd_workspace_bytes(s, accumulate_f32);
-  MLTS_REQUIRE(workspace && workspace_bytes >= need, "mlts_attn_bwd: workspace too small (%lld < %lld)",
+int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
+                  const void* k, const void* v, const void* o, const float* lse, void* dq, const int64_t dq_stride[3],
+                  void* dk, const int64_t dk_stride[3], void* dv, const int64_t dv_stride[3], int accumulate_f32,
+                  void* workspace, int64_t workspace_bytes, hipStream_t st) {
+  MLTS_REQUIRE(dout && q && k && v && o && lse && dq && dk && dv, "%s: null tensor pointer", who);
+  MLTS_REQUIRE(do_stride && dq_stride && dk_stride && dv_stride, "%s: null stride pointer", who);
+  const int64_t need = bwd_min_workspace(s);
+  MLTS_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace too small (%lld < %lld)", who,
                (long long)workspace_bytes, (long long)need);
-  hipStream_t st = static_cast<hipStream_t>(stream);
   AttnBwdParams bp;
   fill_params(bp.a, s, q, k, v, const_cast<void*>(o), const_cast<float*>(lse));
   char* ws = setup_stats(bp.a, s, static_cast<char*>(workspace), st);
@@ -226,21 +217,108 @@ extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const i
   bp.nkt = 0;
   bp.ds_ws = nullptr;
   bp.ds_nkb = bp.ds_nqt = 0;
+  if (uses_mfma(s)) {
+    MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
+                     mlts_aligned16(dq) && mlts_aligned16(dk) && mlts_aligned16(dv),
+                 "%s: tensors must be 16-byte aligned", who);
+    const int es_out = accumulate_f32 ? 4 : 2;
+    MLTS_REQUIRE(strides_aligned(do_stride, 2) && strides_aligned(dq_stride, es_out) &&
+                     strides_aligned(dk_stride, es_out) && strides_aligned(dv_stride, es_out),
+                 "%s: strides must keep rows 16-byte aligned", who);
+    MLTS_REQUIRE(do_stride[2] < kMaxRowStride, "%s: the sequence stride of dout must be below 2^24 elements", who);
+  }
   if (s->Sq > 0) {
     int rc = mlts_attn_delta(dout, do_stride, o, s->o_stride, delta, s->B, s->Hq, s->Sq, s->D, s->dtype, st);
     if (rc != MLTS_OK) return rc;
   }
-  if (uses_mfma(s)) {
-    MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
-                     mlts_aligned16(dq) && mlts_aligned16(dk) && mlts_aligned16(dv),
-                 "mlts_attn_bwd: tensors must be 16-byte aligned");
-    const int es_out = accumulate_f32 ? 4 : 2;
-    MLTS_REQUIRE(strides_aligned(do_stride, 2) && strides_aligned(dq_stride, es_out) &&
-                     strides_aligned(dk_stride, es_out) && strides_aligned(dv_stride, es_out),
-                 "mlts_attn_bwd: strides must keep rows 16-byte aligned");
-    return mlts_attn_bwd_bf16(bp, s->D, s->mask_mode, ws, st);
+  if (!uses_mfma(s)) return mlts_attn_generic_bwd(bp, s->D, s->dtype, s->mask_mode, st);
+  void* lse2_ws = ws;
+  ws += mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);
+  const int64_t ds_bytes = ds_handover_bytes(s, accumulate_f32);
+  void* ds_ws = ds_bytes > 0 && workspace_bytes >= need + ds_bytes ? ws : nullptr;
+  return attn_bwd_bf16(bp, s->D, s->mask_mode, lse2_ws, ds_ws, st);
+}
+
+}  // namespace
+
+// ---- tile statistics ------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restrict__ pos, const int32_t* __restrict__ seq,
+                                                        int S, int ntiles, int4* __restrict__ out) {
+  const int t = blockIdx.x % ntiles, b = blockIdx.x / ntiles;
+  const int i = t * kAttnTile + threadIdx.x;
+  int pmin = 0x7fffffff, pmax = -0x7fffffff - 1, smin = 0x7fffffff, smax = -0x7fffffff - 1;
+  if (i < S) {
+    const int pp = pos[static_cast<int64_t>(b) * S + i], ss = seq[static_cast<int64_t>(b) * S + i];
+    pmin = pmax = pp;
+    smin = smax = ss;
   }
-  return mlts_attn_generic_bwd(bp, s->D, s->dtype, s->mask_mode, st);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    pmin = min(pmin, __shfl_xor(pmin, o, 64));
+    pmax = max(pmax, __shfl_xor(pmax, o, 64));
+    smin = min(smin, __shfl_xor(smin, o, 64));
+    smax = max(smax, __shfl_xor(smax, o, 64));
+  }
+  if (threadIdx.x == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
+}
+
+
+void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
+  const int ntiles = (S + kAttnTile - 1) / kAttnTile;
+  if (B * ntiles == 0) return;
+  hipLaunchKernelGGL(tile_stats_kernel, dim3(B * ntiles), dim3(64), 0, st, pos, seq, S, ntiles, out);
+}
+
+extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return shape_problem(s); }
+
+extern "C" int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s) {
+  if (shape_problem(s)) return -1;
+  return stats_bytes(s);
+}
+
+extern "C" int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32) {
+  (void)accumulate_f32;
+  if (shape_problem(s)) return -1;
+  return bwd_min_workspace(s);
+}
+
+extern "C" int64_t mlts_attn_bwd_ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32) {
+  if (shape_problem(s)) return -1;
+  return ds_handover_bytes(s, accumulate_f32);
+}
+
+extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o, float* lse,
+                             void* workspace, int64_t workspace_bytes, mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_fwd: %s", why);
+  if (s->B == 0 || s->Sq == 0) return MLTS_OK;
+  MLTS_REQUIRE(q && o && lse, "mlts_attn_fwd: q, o, lse must be non-null");
+  MLTS_REQUIRE(s->Sk == 0 || (k && v), "mlts_attn_fwd: k, v must be non-null");
+  const int64_t need = stats_bytes(s);
+  MLTS_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), "mlts_attn_fwd: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  AttnParams p;
+  fill_params(p, s, q, k, v, o, lse);
+  if (uses_mfma(s)) {
+    MLTS_REQUIRE(mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) && mlts_aligned16(o),
+                 "mlts_attn_fwd: q, k, v, o must be 16-byte aligned");
+    setup_stats(p, s, static_cast<char*>(workspace), st);
+    return mlts_attn_fwd_bf16_dma(p, s->D, s->mask_mode, st);
+  }
+  return mlts_attn_generic_fwd(p, s->D, s->dtype, s->mask_mode, st);
+}
+
+extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
+                             const void* k, const void* v, const void* o, const float* lse, void* dq,
+                             const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,
+                             const int64_t dv_stride[3], int accumulate_f32, void* workspace, int64_t workspace_bytes,
+                             mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_bwd: %s", why);
+  if (s->B == 0 || (s->Sq == 0 && s->Sk == 0)) return MLTS_OK;
+  return attn_bwd_impl("mlts_attn_bwd", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv, dv_stride,
+                       accumulate_f32, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk, const int64_t o_blk_stride[3],

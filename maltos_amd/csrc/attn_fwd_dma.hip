@@ -98,7 +98,8 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   constexpr int KS = C::KS, DB = C::DB, RB = C::RB, CPR = C::CPR, TILE_BYTES = C::TILE_BYTES, STAGE_BYTES = C::STAGE_BYTES,
                 PPW = C::PPW, LOADS_PER_TILE = C::LOADS_PER_TILE;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
   const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
 
   // Longest (last) q-tiles first across the whole grid: with causal masks the work per q-tile varies 16:1 and
@@ -168,23 +169,40 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 
   // ---- DMA loader: this wavefront moves PPW 1 KiB pieces of the K tile and of the V tile; piece n holds rows
   // n * 64 / CPR ..; lane L -> row n * 64 / CPR + L / CPR, stored chunk L % CPR, source chunk (L % CPR) ^ swz(row) ----
+  // Addresses are a wave-uniform tile base (scalar arithmetic) plus a tile-invariant lane offset, so a tile's loads cost
+  // four instructions and almost no vector arithmetic; only a tile that reaches past Sk clamps its rows.
   int ld_row[PPW], ld_col[PPW];
+  uint32_t ld_koff[PPW], ld_voff[PPW];
 #pragma unroll
   for (int n = 0; n < PPW; ++n) {
     const int row = (wave * PPW + n) * (64 / CPR) + lane / CPR;
     ld_row[n] = row;
     ld_col[n] = ((lane % CPR) ^ swz<D>(row & 15)) * 8;
+    ld_koff[n] = static_cast<uint32_t>(row * static_cast<int>(p.ks[2]) + ld_col[n]) * 2u;
+    ld_voff[n] = static_cast<uint32_t>(row * static_cast<int>(p.vs[2]) + ld_col[n]) * 2u;
   }
+  const unsigned char* Kb = reinterpret_cast<const unsigned char*>(K);
+  const unsigned char* Vb = reinterpret_cast<const unsigned char*>(V);
   auto issue_tile = [&](int j, int stage) {
     const int kv0 = j * BN;
-    unsigned char* sbase = smem + stage * STAGE_BYTES;
+    unsigned char* sbase = smem + stage * STAGE_BYTES + wave * PPW * 1024;
+    if (kv0 + BN <= p.Sk) {
+      const unsigned char* kt = Kb + static_cast<int64_t>(kv0) * p.ks[2] * 2;
+      const unsigned char* vt = Vb + static_cast<int64_t>(kv0) * p.vs[2] * 2;
 #pragma unroll
-    for (int n = 0; n < PPW; ++n) {
-      const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
-      const bf16_t* ksrc = K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n];
-      const bf16_t* vsrc = V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n];
-      __builtin_amdgcn_global_load_lds(MLTS_GLB(ksrc), MLTS_LDS(sbase + (wave * PPW + n) * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(MLTS_GLB(vsrc), MLTS_LDS(sbase + TILE_BYTES + (wave * PPW + n) * 1024), 16, 0, 0);
+      for (int n = 0; n < PPW; ++n) {
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(kt + ld_koff[n]), MLTS_LDS(sbase + n * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(vt + ld_voff[n]), MLTS_LDS(sbase + TILE_BYTES + n * 1024), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < PPW; ++n) {
+        const int r = min(kv0 + ld_row[n], p.Sk - 1);  // rows past the end repeat the last key; their scores are masked
+        const bf16_t* ksrc = K + static_cast<int64_t>(r) * p.ks[2] + ld_col[n];
+        const bf16_t* vsrc = V + static_cast<int64_t>(r) * p.vs[2] + ld_col[n];
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(ksrc), MLTS_LDS(sbase + n * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(vsrc), MLTS_LDS(sbase + TILE_BYTES + n * 1024), 16, 0, 0);
+      }
     }
   };
 
