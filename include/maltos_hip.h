@@ -113,6 +113,19 @@ int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_s
                   const int64_t dv_stride[3], int accumulate_f32, void* workspace, int64_t workspace_bytes,
                   mlts_stream_t stream);
 
+/* mlts_attn_bwd for callers that cannot allocate device memory or bring a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as mlts_attn_bwd with a workspace of exactly mlts_attn_bwd_workspace_bytes (the recomputing backward); the
+ * workspace is a buffer of MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE bytes inside the library image, one copy per GPU, held
+ * until the process ends.  Shapes whose workspace is larger (about B * Hq * Sq > 1 M query rows) are rejected with
+ * MLTS_ERR_INVALID.  No hipMalloc / hipFree is made.  All calls on one GPU share that buffer: calls that may overlap
+ * on one GPU (different streams, different threads) race; serialise them or use mlts_attn_bwd. */
+#define MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE (8 << 20)
+int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
+                          const void* k, const void* v, const void* o, const float* lse, void* dq,
+                          const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,
+                          const int64_t dv_stride[3], int accumulate_f32, mlts_stream_t stream);
+
 /* Log-sum-exp merge of one block into the running fp32 state, rows [q_off, q_off + q_len):
  *   lse' = logaddexp(lse, lse_b); out' = out * exp(lse - lse') + out_b * exp(lse_b - lse'),
  * with exp(-inf - x) := 0 (a row where both are -inf becomes 0 with lse -inf).  Replaces

@@ -73,6 +73,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         C.c_int,
         [_SHAPE_P, _P, _I64P, _P, _P, _P, _P, _P, _P, _I64P, _P, _I64P, _P, _I64P, C.c_int, _P, C.c_int64, _P],
     ),
+    "mlts_attn_bwd_noalloc": (
+        C.c_int,
+        [_SHAPE_P, _P, _I64P, _P, _P, _P, _P, _P, _P, _I64P, _P, _I64P, _P, _I64P, C.c_int, _P],
+    ),
     "mlts_attn_merge": (
         C.c_int,
         [_P, _P, _P, _I64P, C.c_int32, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P],

@@ -1,6 +1,8 @@
 // C-ABI entry points for attention: argument validation on the host, workspace carving, kernel
 // selection (bf16 head_dim 64/128 -> MFMA kernels, everything else -> generic fp32-ALU kernels) and
 // the log-sum-exp block merge.
+#include <mutex>
+
 #include "attn_common.hpp"
 
 int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st);                        // attn_fwd_dma.hip
@@ -239,6 +241,37 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
   return attn_bwd_bf16(bp, s->D, s->mask_mode, lse2_ws, ds_ws, st);
 }
 
+// ---- scratch of the entry point that allocates nothing --------------------------------------------------------
+// Device memory that belongs to the library image: every GPU the library runs on holds its own copy at its own
+// address until the process ends.  Host code never uses the array's name as an address; the per-device address is
+// looked up once (hipGetSymbolAddress with that device current) and kept in g_scratch_addr.
+constexpr int64_t kScratchBytes = MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE;
+__device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_addr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_for_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    mlts_set_error("mlts_attn_bwd_noalloc: cannot identify the current device (%s)", hipGetErrorString(e));
+    return MLTS_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_addr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      mlts_set_error("mlts_attn_bwd_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return MLTS_ERR_LAUNCH;
+    }
+    g_scratch_addr[dev] = ptr;
+  }
+  *out = g_scratch_addr[dev];
+  return MLTS_OK;
+}
+
 }  // namespace
 
 // ---- tile statistics ------------------------------------------------------------------------
@@ -319,6 +352,26 @@ extern "C" int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const i
   if (s->B == 0 || (s->Sq == 0 && s->Sk == 0)) return MLTS_OK;
   return attn_bwd_impl("mlts_attn_bwd", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv, dv_stride,
                        accumulate_f32, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
+                                     const void* k, const void* v, const void* o, const float* lse, void* dq,
+                                     const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,
+                                     const int64_t dv_stride[3], int accumulate_f32, mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_bwd_noalloc: %s", why);
+  if (s->B == 0 || (s->Sq == 0 && s->Sk == 0)) return MLTS_OK;
+  const int64_t need = bwd_min_workspace(s);
+  MLTS_REQUIRE(need <= kScratchBytes,
+               "mlts_attn_bwd_noalloc: this shape needs %lld bytes of workspace, the built-in scratch holds %lld "
+               "(about B*Hq*Sq <= %lld query rows); use mlts_attn_bwd with a caller workspace",
+               (long long)need, (long long)kScratchBytes, (long long)(kScratchBytes / 8 - 64));
+  void* ws = nullptr;
+  int rc = scratch_for_current_device(&ws);
+  if (rc != MLTS_OK) return rc;
+  // exactly `need` bytes are offered, so the dS hand-over (which needs more) is never taken
+  return attn_bwd_impl("mlts_attn_bwd_noalloc", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv,
+                       dv_stride, accumulate_f32, ws, need, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk, const int64_t o_blk_stride[3],
