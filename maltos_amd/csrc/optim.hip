@@ -28,7 +28,10 @@ __device__ __forceinline__ float clip_coef(const AdamArgs& a) {
 }
 
 __device__ __forceinline__ void adam_update(float& p, float g, float& m, float& v, const AdamArgs& a, float c) {
+  // rounded product, never contracted into the arithmetic below: clipping inside this kernel then gives the very bits of
+  // a separate scaling pass over the gradients followed by an unclipped step, whichever way a caller clips
   g *= c;
+  asm volatile("" : "+v"(g));
   p -= a.lr * a.weight_decay * p;
   m = m + (1.0f - a.beta1) * (g - m);
   v = a.beta2 * v + (1.0f - a.beta2) * g * g;

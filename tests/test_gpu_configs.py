@@ -108,6 +108,9 @@ def test_cfg2_dense_causal_bf16_full_size(dev):
             lib = _sdpa_math_fp32(qf.detach(), kf.detach(), vf.detach())
             assert (lib - want_o).abs().max() <= 1e-5
     print(f"cfg2 max abs errors: {worst}")
+    # the stated bar without the half-ulp allowance: it holds outright at this configuration
+    for name, err in worst.items():
+        assert err <= 2e-2, f"{name}: max abs error {err:.4f} above 2e-2"
     # size-independent invariants: softmax rows sum to one
     ones = torch.ones_like(v)
     o1 = ops.attention(q, k, ones, mask_mode=ops.MASK_CAUSAL)
@@ -171,7 +174,7 @@ def test_cfg3_packed_documents_gqa_bf16_full_size(dev):
 
 
 # ------------------------------------------------------------------ cfg4
-@pytest.mark.parametrize("rank", [0, 2])
+@pytest.mark.parametrize("rank", [0, 1, 2, 3])
 def test_cfg4_zigzag_ring_rank_share_bf16_full_size(dev, rank):
     W, H, S_loc, D = 4, 16, 8192, 128
     total = W * S_loc
@@ -232,12 +235,15 @@ def test_cfg5_llama50m_bf16_train_step(dev):
     opt.zero_grad(set_to_none=True)
     # oracle: (a) fp32 evaluation of the bf16-rounded network, (b) the reference-style eager bf16 evaluation
     results = {}
+    fp32_grads = None
     for tag, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
         leaves = OrderedDict((n, p.to(dev).to(torch.bfloat16).to(dtype).requires_grad_(True)) for n, p in params.items())
         logits = ol.forward(leaves, cfg, input_ids)
         ref_loss = F.cross_entropy(logits.float().view(-1, cfg.vocab_size), labels.view(-1))
         ref_loss.backward()
         results[tag] = (ref_loss.item(), oo.global_grad_norm([p.grad for p in leaves.values()]))
+        if tag == "fp32":
+            fp32_grads = OrderedDict((n, p.grad.detach()) for n, p in leaves.items())
         del logits, leaves
     want_loss, want_norm = results["fp32"]
     print(f"cfg5 loss hip={loss.item():.6f} fp32={want_loss:.6f} bf16-eager={results['bf16'][0]:.6f}; "
@@ -254,3 +260,29 @@ def test_cfg5_llama50m_bf16_train_step(dev):
     assert moved > 0
     for mp, p in zip(opt.master_params, model.parameters()):
         assert torch.equal(p.detach(), mp.detach().to(torch.bfloat16))
+    # post-step fp32 masters against the oracle's step (clip at 1.0 on the fp32 gradients, then stock AdamW) on a
+    # sample of tensors.  AdamW's first step is lr * g / (|g| + eps): it only keeps the SIGN of each gradient element,
+    # so the two paths agree to fp32 rounding wherever the bf16 pipeline's gradient noise does not flip a sign, and
+    # differ by 2 * lr where it does (elements with |g| far below the typical magnitude).
+    coef = min(1.0, oo.clip_coefficient(want_norm, 1.0))
+    masters = dict(zip((n for n, _ in model.named_parameters()), opt.master_params))
+    lr = 3e-4
+    for name in ("embed_tokens.weight", "layers.0.self_attn.q_proj.weight", "layers.3.mlp.gate_proj.weight",
+                 "layers.7.mlp.down_proj.weight", "layers.7.input_layernorm.weight", "norm.weight", "lm_head.weight"):
+        start = params[name].to(dev).to(torch.bfloat16).float()
+        want = torch.nn.Parameter(start.clone())
+        want.grad = fp32_grads[name] * coef
+        torch.optim.AdamW([want], lr=lr, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1).step()
+        diff = (masters[name].detach() - want.detach()).abs()
+        touched = fp32_grads[name].abs() > 0          # rows of the embedding no token selected keep g = 0 on both sides
+        flipped = (diff > 0.5 * lr) & touched
+        assert diff.max() <= 2 * lr * 1.001 + 1e-7, f"{name}: {diff.max().item():.3e}"
+        assert flipped.float().mean() <= 0.05, f"{name}: {flipped.float().mean().item():.4f} of the elements moved the other way"
+        # elsewhere the step is lr * g / (|g| + eps) on both sides: lr * sign(g) up to eps / |g| (the clipped gradients of
+        # the embedding rows are only 10^2..10^3 eps), so within 5 % of lr for all but a percent of the elements, those whose gradient
+        # nearly cancels in one of the two evaluations
+        same = touched & ~flipped
+        off = (diff > 0.05 * lr) & same
+        assert off.float().sum() <= 1e-2 * same.float().sum(), f"{name}: {off.float().sum().item() / same.float().sum().item():.5f}"
+        print(f"cfg5 masters {name}: sign flips {flipped.float().mean().item():.5f}, others off by > 0.05 lr: {off.float().mean().item():.6f}, "
+              f"median diff {diff[same].median().item():.2e}")

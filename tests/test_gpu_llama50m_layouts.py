@@ -1,0 +1,165 @@
+"""LLaMA-50M (the fifth benchmark configuration's shapes) in the two optimizer layouts, and under activation
+checkpointing.
+
+  * flat layout (MasterWeightsOptimizer over the model's parameters) vs ZeRO-1 layout (Zero1FlatBuffers: reverse-order
+    25 MiB buckets, flat data / grad buffers, per-bucket local shards).  Both run the same kernels on the same numbers,
+    only at other addresses: after one step from identical weights the bf16 gradients, the norm and the fp32 masters
+    are compared bit for bit, and the test names the first tensor that differs if any does.  Over several steps the
+    two trajectories are bounded against each other.
+  * ZeRO-1 layout against the library: stock torch.optim.AdamW + torch.nn.utils.clip_grad_norm_ on fp32 shadow copies
+    fed with the same bf16 gradients (the recipe of runtime/optim.py:43-71 and runtime/plugins/zero_common.py:307-351).
+  * non-reentrant activation checkpointing of every decoder layer (models/llama.py:278-289) gives the gradients of the
+    plain forward, with and without weight-gradient accumulation into bound buffers.
+"""
+import copy
+from collections import OrderedDict
+
+import pytest
+import torch
+
+from maltos_amd.grad_clip import clip_grad_norm_
+from maltos_amd.llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
+from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
+from maltos_amd.zero1 import Zero1FlatBuffers
+
+pytestmark = pytest.mark.gpu
+
+CFG5 = dict(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8, num_attention_heads=8,
+            max_position_embeddings=2048, rms_norm_eps=1e-5, rope_theta=10000.0)
+HP = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+
+
+def _model(dev, layers=8):
+    torch.manual_seed(1234)
+    model = LlamaForCausalLM(LlamaConfig(**{**CFG5, "num_hidden_layers": layers}))
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() >= 2:
+                p.normal_(0.0, 0.02)
+    return model.to(dev).to(torch.bfloat16)
+
+
+def _batch(dev, seed=1234, rows=8, seq=2048):
+    ids = torch.randint(0, 32000, (rows, seq + 1), generator=torch.Generator().manual_seed(seed)).to(dev)
+    return {"input_ids": ids[:, :-1].contiguous(), "labels": ids[:, 1:].contiguous()}
+
+
+def _factory(ps):
+    return MasterWeightsOptimizer(ps, optimizer_factory=lambda q: FusedAdamW(q, **HP))
+
+
+@pytest.mark.parametrize("accumulate", [False, True], ids=["autograd-accumulation", "accumulate-into-buffers"])
+def test_flat_and_zero1_layouts_take_the_same_step(dev, accumulate):
+    flat_model = _model(dev)
+    zero_model = copy.deepcopy(flat_model)
+    if accumulate:
+        set_grad_accumulation_into_buffers(flat_model)
+        set_grad_accumulation_into_buffers(zero_model)
+    opt = _factory(list(flat_model.parameters()))
+    z = Zero1FlatBuffers(zero_model, optimizer_factory=_factory, bucket_mb_size=25)
+    names = [n for n, _ in flat_model.named_parameters()]
+    history = []
+    for step in range(4):
+        batch = _batch(dev, seed=1234 + step)
+        loss_f = flat_model(batch)
+        loss_f.backward()
+        z.reset_grads()
+        loss_z = zero_model(batch)
+        loss_z.backward()
+        if step == 0:
+            # identical weights, identical batch: the same numbers at other addresses
+            assert loss_f.item() == loss_z.item()
+            for n, pf, pz in zip(names, flat_model.parameters(), zero_model.parameters()):
+                assert torch.equal(pf.grad, pz.grad), f"first differing bf16 gradient: {n}"
+        norm_f = clip_grad_norm_(opt, 1.0)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        norm_z = z.step(1.0)
+        history.append((loss_f.item(), loss_z.item(), norm_f, norm_z))
+        if step == 0:
+            # fp64 sums of the same squares in another order (the buckets are in reverse parameter order)
+            assert abs(norm_f - norm_z) <= 1e-12 * norm_f
+            for n, pf, pz in zip(names, flat_model.parameters(), zero_model.parameters()):
+                assert torch.equal(pf.detach(), pz.detach()), f"first differing parameter after the step: {n}"
+    print("loss/norm history (flat, zero1):", history)
+    # later steps start from bit-equal weights as long as every step is bit-equal; they are
+    for lf, lz, nf, nz in history:
+        assert lf == lz and abs(nf - nz) <= 1e-12 * nf
+
+
+def test_device_side_clip_takes_the_same_steps_as_host_side_clip(dev):
+    """clip_grad_norm_fused_ (norm stays on the device, the AdamW kernel applies the coefficient) against clip_grad_norm_
+    (host reads the norm, a scaling pass, then the step): bit-equal masters over steps that do and do not clip."""
+    from maltos_amd.grad_clip import clip_grad_norm_fused_
+
+    a = _model(dev)
+    b = copy.deepcopy(a)
+    opt_a, opt_b = _factory(list(a.parameters())), _factory(list(b.parameters()))
+    clipped = 0
+    for step in range(7):
+        batch = _batch(dev, seed=1234)
+        a(batch).backward()
+        b(batch).backward()
+        norm = clip_grad_norm_(opt_a, 1.0)
+        opt_a.step()
+        opt_a.zero_grad(set_to_none=True)
+        sq = clip_grad_norm_fused_(opt_b, 1.0)
+        opt_b.step()
+        opt_b.zero_grad(set_to_none=True)
+        clipped += norm > 1.0
+        assert abs(float(sq.sqrt()) - norm) <= 1e-12 * norm
+        for x, y in zip(opt_a.master_params, opt_b.master_params):
+            assert torch.equal(x.detach(), y.detach()), f"step {step} (norm {norm:.3f})"
+    assert clipped >= 1
+
+
+def test_zero1_layout_matches_library_adamw_and_clip(dev):
+    model = _model(dev, layers=2)
+    z = Zero1FlatBuffers(model, optimizer_factory=_factory, bucket_mb_size=25)
+    params = list(model.parameters())
+    shadow = [torch.nn.Parameter(p.detach().float().clone()) for p in params]
+    lib = torch.optim.AdamW(shadow, **HP)
+    for step in range(3):
+        z.reset_grads()
+        model(_batch(dev, seed=77 + step, rows=2, seq=512)).backward()
+        for s, p in zip(shadow, params):
+            s.grad = p.grad.detach().float().clone()
+        want_norm = torch.nn.utils.clip_grad_norm_(shadow, 1.0).item()
+        lib.step()
+        got_norm = z.step(1.0)
+        assert abs(got_norm - want_norm) <= 1e-5 * want_norm
+        masters = {}
+        inner_masters = z.optimizer.master_params
+        for bucket, mp in zip(z.buckets, inner_masters):
+            cursor = 0
+            for p in bucket.params:
+                masters[id(p)] = mp.detach()[cursor:cursor + p.numel()].view_as(p)
+                cursor += p.numel()
+        for s, p in zip(shadow, params):
+            torch.testing.assert_close(masters[id(p)], s.detach(), rtol=1e-4, atol=1e-7)
+            assert torch.equal(p.detach(), masters[id(p)].to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("accumulate", [False, True], ids=["autograd-accumulation", "accumulate-into-buffers"])
+def test_non_reentrant_checkpointing_gives_the_same_gradients(dev, accumulate):
+    from torch.utils.checkpoint import checkpoint
+
+    plain = _model(dev, layers=3)
+    ckpt = copy.deepcopy(plain)
+    opts = []
+    for m in (plain, ckpt):
+        if accumulate:
+            set_grad_accumulation_into_buffers(m)
+            opts.append(_factory(list(m.parameters())))   # binds every gradient to a view of a flat buffer
+    for layer in ckpt.layers:
+        inner = layer.forward
+        layer.forward = (lambda fwd: lambda *a, **kw: checkpoint(fwd, *a, use_reentrant=False, **kw))(inner)
+    batch = _batch(dev, seed=5, rows=2, seq=1024)
+    for rep in range(2):   # twice: the second backward finds gradients already in place
+        loss_p = plain(batch)
+        loss_p.backward()
+        loss_c = ckpt(batch)
+        loss_c.backward()
+        assert loss_p.item() == loss_c.item()
+        for (n, a), b in zip(plain.named_parameters(), ckpt.parameters()):
+            assert torch.equal(a.grad, b.grad), f"rep {rep}: {n}"
