@@ -313,14 +313,10 @@ int launch(AttnBwdParams bp, hipStream_t st) {
   auto kern = attn_bwd_dq_ds_kernel<D, CAUSAL>;
   constexpr int lds_bytes = DsCfg<D>::LDS_BYTES;
   static_assert(lds_bytes >= WAVES * 32 * DsCfg<D>::RB, "the epilogue needs 32 rows per wavefront");
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-      return MLTS_ERR_LAUNCH;
-    }
-    configured = true;
+  static MltsLdsOptIn lds_opt_in;
+  if (hipError_t e = lds_opt_in.reserve(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) {
+    mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    return MLTS_ERR_LAUNCH;
   }
   bp.a.nqt = (bp.a.Sq + BM - 1) / BM;
   const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * bp.a.Hq;

@@ -467,14 +467,10 @@ template <int D, int MODE>
 int launch(AttnBwdParams bp, hipStream_t st) {
   auto kern = attn_bwd_dq_tr_kernel<D, MODE>;
   constexpr int lds_bytes = DqCfg<D>::LDS_BYTES;
-  static bool configured = false;
-  if (!configured && lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-      return MLTS_ERR_LAUNCH;
-    }
-    configured = true;
+  static MltsLdsOptIn lds_opt_in;
+  if (hipError_t e = lds_opt_in.reserve(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) {
+    mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    return MLTS_ERR_LAUNCH;
   }
   bp.a.nqt = (bp.a.Sq + BM - 1) / BM;
   const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * bp.a.Hq;

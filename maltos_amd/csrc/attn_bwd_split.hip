@@ -740,14 +740,10 @@ template <int D, int MODE>
 int launch(const AttnBwdParams& bp, const float* lse2, hipStream_t st) {
   auto kern = attn_bwd_dkdv_split_kernel<D, MODE>;
   constexpr int lds_bytes = SplitCfg<D>::LDS_BYTES;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-      return MLTS_ERR_LAUNCH;
-    }
-    configured = true;
+  static MltsLdsOptIn lds_opt_in;
+  if (hipError_t e = lds_opt_in.reserve(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) {
+    mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    return MLTS_ERR_LAUNCH;
   }
   const int64_t blocks = static_cast<int64_t>(bp.nkt) * bp.a.B * bp.a.Hkv;
   if (blocks > 0) {

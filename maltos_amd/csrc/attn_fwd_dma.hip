@@ -530,14 +530,10 @@ template <int D, int MODE>
 int launch(AttnParams p, hipStream_t st) {
   auto kern = attn_fwd_dma_kernel<D, MODE>;
   constexpr int lds_bytes = FwdCfg<D>::LDS_BYTES;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-      return MLTS_ERR_LAUNCH;
-    }
-    configured = true;
+  static MltsLdsOptIn lds_opt_in;
+  if (hipError_t e = lds_opt_in.reserve(reinterpret_cast<const void*>(kern), lds_bytes); e != hipSuccess) {
+    mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+    return MLTS_ERR_LAUNCH;
   }
   p.nqt = (p.Sq + BM - 1) / BM;
   const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * p.Hq;

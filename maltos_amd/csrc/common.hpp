@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <stdarg.h>
 
+#include <mutex>
+
 #include "../../include/maltos_hip.h"
 
 typedef __bf16 bf16_t;
@@ -32,6 +34,17 @@ struct MltsKernelTimer {
   hipStream_t stream_;
   hipEvent_t start_;
   bool active_;
+};
+
+// One-time opt-in of a kernel to more than 48 KiB of dynamic LDS; safe when several host threads make their first launch
+// of that kernel at once.  One instance per kernel instantiation (a function-local static).
+struct MltsLdsOptIn {
+  std::once_flag once;
+  hipError_t err = hipSuccess;
+  hipError_t reserve(const void* kernel, int bytes) {
+    std::call_once(once, [&] { err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes); });
+    return err;
+  }
 };
 
 #define MLTS_REQUIRE(cond, ...)        \

@@ -230,7 +230,8 @@ def _rmsnorm_fwd(x, w, eps):
     x2 = x.contiguous().view(-1, hidden)
     y = torch.empty_like(x2)
     rstd = torch.empty(x2.size(0), dtype=torch.float32, device=x.device)
-    _lib.check(_lib.lib().mlts_rmsnorm_fwd(_p(x2), _p(w.contiguous()), _p(y), _p(rstd), x2.size(0), hidden, float(eps),
+    w = w.contiguous()   # kept in a local until after the launch
+    _lib.check(_lib.lib().mlts_rmsnorm_fwd(_p(x2), _p(w), _p(y), _p(rstd), x2.size(0), hidden, float(eps),
                                            _dtype_code(x), _stream()))
     return y.view(x.shape), rstd
 
@@ -247,7 +248,8 @@ def _rmsnorm_bwd(dy, x, w, rstd):
     L = _lib.lib()
     ws_bytes = L.mlts_rmsnorm_bwd_workspace_bytes(x2.size(0), hidden)
     ws = _workspace(ws_bytes, x.device)
-    _lib.check(L.mlts_rmsnorm_bwd(_p(dy2), _p(x2), _p(w.contiguous()), _p(rstd), _p(dx), _p(dw), _p(ws), ws_bytes,
+    w = w.contiguous()
+    _lib.check(L.mlts_rmsnorm_bwd(_p(dy2), _p(x2), _p(w), _p(rstd), _p(dx), _p(dw), _p(ws), ws_bytes,
                                   x2.size(0), hidden, _dtype_code(x), _stream()))
     return dx.view(x.shape), dw
 
@@ -264,7 +266,8 @@ def _add_rmsnorm_fwd(x, res, w, eps):
     h = torch.empty_like(x2)
     y = torch.empty_like(x2)
     rstd = torch.empty(x2.size(0), dtype=torch.float32, device=x.device)
-    _lib.check(_lib.lib().mlts_add_rmsnorm_fwd(_p(x2), _p(r2), _p(h), _p(w.contiguous()), _p(y), _p(rstd), x2.size(0), hidden,
+    w = w.contiguous()
+    _lib.check(_lib.lib().mlts_add_rmsnorm_fwd(_p(x2), _p(r2), _p(h), _p(w), _p(y), _p(rstd), x2.size(0), hidden,
                                                float(eps), _dtype_code(x), _stream()))
     return h.view(x.shape), y.view(x.shape), rstd
 
@@ -282,7 +285,8 @@ def _add_rmsnorm_bwd(dy, dres, h, w, rstd):
     L = _lib.lib()
     ws_bytes = L.mlts_rmsnorm_bwd_workspace_bytes(h2.size(0), hidden)
     ws = _workspace(ws_bytes, h.device)
-    _lib.check(L.mlts_add_rmsnorm_bwd(_p(dy2), _p(h2), _p(w.contiguous()), _p(rstd), _p(dr2), _p(dx), _p(dw), _p(ws), ws_bytes,
+    w = w.contiguous()
+    _lib.check(L.mlts_add_rmsnorm_bwd(_p(dy2), _p(h2), _p(w), _p(rstd), _p(dr2), _p(dx), _p(dw), _p(ws), ws_bytes,
                                       h2.size(0), hidden, _dtype_code(h), _stream()))
     return dx.view(h.shape), dw
 
@@ -301,8 +305,9 @@ def _rope(x, cos, sin, positions, position_offset, inverse):
     pos32 = None
     if positions is not None:
         pos32 = _ids32(positions, B, S, "position_ids")
-    _lib.check(_lib.lib().mlts_rope(_p(x), strides3(x.stride()[:3]), _p(y), strides3(y.stride()[:3]), _p(cos.contiguous()),
-                                    _p(sin.contiguous()), cos.size(0), _p(pos32), int(position_offset), B, H, S, D,
+    cos, sin = cos.contiguous(), sin.contiguous()
+    _lib.check(_lib.lib().mlts_rope(_p(x), strides3(x.stride()[:3]), _p(y), strides3(y.stride()[:3]), _p(cos),
+                                    _p(sin), cos.size(0), _p(pos32), int(position_offset), B, H, S, D,
                                     _dtype_code(x), int(bool(inverse)), _stream()))
     return y
 

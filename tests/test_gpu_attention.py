@@ -160,6 +160,14 @@ def test_empty_and_error_cases(dev):
     q = torch.randn(1, 2, 4, 64, device=dev)
     o, lse = ops.attention_forward(q, kv[:, :, :0], kv[:, :, :0], mask_mode=ops.MASK_NONE)  # no keys: zeros, -inf
     assert not o.any() and (lse == float("-inf")).all()
+    # the same on the bf16 MFMA kernels (head_dim 64 and 128), forward and backward
+    for D in (64, 128):
+        qb = torch.randn(1, 2, 40, D, device=dev).bfloat16()
+        kb = torch.randn(1, 2, 0, D, device=dev).bfloat16()
+        o, lse = ops.attention_forward(qb, kb, kb, mask_mode=ops.MASK_CAUSAL)
+        assert o.dtype == torch.bfloat16 and not o.any() and (lse == float("-inf")).all()
+        dq, dk, dv = ops.attention_backward(torch.ones_like(qb), qb, kb, kb, o, lse, mask_mode=ops.MASK_CAUSAL)
+        assert not dq.any() and dk.shape == kb.shape and dv.shape == kb.shape
     with pytest.raises(ValueError):
         ops.attention(q, kv.half(), kv.half())
     with pytest.raises(ValueError):

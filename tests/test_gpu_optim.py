@@ -242,3 +242,35 @@ def test_linear_accumulates_weight_grad_into_bound_buffer(dev, rows, out_f, in_f
     xi = x.clone().requires_grad_(True)
     fused(xi).backward(dy)
     assert fused.weight.grad is not None and (fused.weight.grad.double() - (exact - start.double())).abs().max() < 0.5
+
+
+def test_unused_parameter_is_skipped_in_the_per_parameter_layout(dev):
+    """A parameter that received no gradient: the reference leaves its master gradient at None and the inner optimizer
+    skips it (runtime/optim.py:46-50).  MasterWeightsOptimizer(flat=False) does the same; the flat layout (the default)
+    binds every gradient to a zeroed buffer, so there the parameter is stepped with a zero gradient (weight decay and
+    moment decay still apply) -- the documented difference."""
+    used = nn.Parameter(torch.randn(8, 16, device=dev).bfloat16())
+    unused = nn.Parameter(torch.randn(4, 16, device=dev).bfloat16())
+    shadow = [used.detach().float().clone().requires_grad_(True), unused.detach().float().clone().requires_grad_(True)]
+    lib = torch.optim.AdamW(shadow, **HP)
+    opt = MasterWeightsOptimizer([used, unused], optimizer_factory=lambda ps: FusedAdamW(ps, **HP), flat=False)
+    before = unused.detach().clone()
+    for _ in range(2):
+        (used.float() ** 2).sum().backward()
+        shadow[0].grad = used.grad.detach().float().clone()
+        assert unused.grad is None
+        opt.step()
+        lib.step()
+        opt.zero_grad(set_to_none=True)
+        lib.zero_grad(set_to_none=True)
+    assert torch.equal(unused.detach(), before)                      # never touched, like the library's
+    torch.testing.assert_close(opt.master_params[0].detach(), shadow[0].detach(), rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(opt.master_params[1].detach(), shadow[1].detach(), rtol=0, atol=0)
+    # the flat layout steps it with a zero gradient: only the decoupled weight decay moves it
+    used2 = nn.Parameter(used.detach().clone())
+    unused2 = nn.Parameter(before.clone())
+    flat = MasterWeightsOptimizer([used2, unused2], optimizer_factory=lambda ps: FusedAdamW(ps, **HP), flat=True)
+    (used2.float() ** 2).sum().backward()
+    flat.step()
+    want = before.float() * (1 - HP["lr"] * HP["weight_decay"])
+    torch.testing.assert_close(flat.master_params[1].detach(), want, rtol=1e-6, atol=1e-8)

@@ -59,6 +59,25 @@ def test_entry_points_validate_before_launch():
     assert L.mlts_attn_supports(ctypes.byref(shape)) is None
     assert L.mlts_attn_fwd_workspace_bytes(ctypes.byref(shape)) == 0
     assert L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 0) >= L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 1) > 0
+    # the workspace is O(B * Hq * Sq); the dS hand-over is a separate, optional amount (head_dim 128 only)
+    assert L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 0) < 64 * 1024
+    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 0) == 0
+    shape.D = 128
+    for arr in (shape.q_stride, shape.k_stride, shape.v_stride, shape.o_stride):
+        arr[0], arr[1], arr[2] = 8 * 3 * 128, 128, 3 * 128
+    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 0) >= 2 * 1 * 3 * 8 * 8
+    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 1) == 0
+    # rows further apart than 2^24 elements are refused (the MFMA kernels address a tile's rows with 32-bit offsets)
+    shape.k_stride[2] = 1 << 24
+    assert b"2^24" in L.mlts_attn_supports(ctypes.byref(shape))
+    shape.k_stride[2] = 3 * 128
+    # the entry point without a workspace refuses shapes beyond its built-in buffer before touching any pointer
+    shape.B, shape.Hq, shape.Hkv, shape.Sq, shape.Sk = 1, 64, 64, 32768, 32768
+    st = (ctypes.c_int64 * 3)(64 * 32768 * 128, 32768 * 128, 128)
+    for arr in (shape.q_stride, shape.k_stride, shape.v_stride, shape.o_stride):
+        arr[0], arr[1], arr[2] = st[0], st[1], st[2]
+    assert L.mlts_attn_bwd_noalloc(ctypes.byref(shape), None, st, None, None, None, None, None, None, st, None, st, None, st, 0, None) == _lib.MLTS_ERR_INVALID
+    assert "built-in scratch" in _lib.last_error()
     with pytest.raises(ValueError):
         _lib.check(_lib.MLTS_ERR_INVALID)
     with pytest.raises(RuntimeError):

@@ -60,3 +60,39 @@ def test_runner_steps_and_reports(dev, tmp_path, extra):
         e = json.loads(eager.read_text())
         assert abs(e["loss_last"] - s["loss_last"]) <= 1e-6 * abs(e["loss_last"])
         assert abs(e["grad_norm_last"] - s["grad_norm_last"]) <= 1e-5 * abs(e["grad_norm_last"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("extra", [["--shards", "tests/golden/tokens_0000*.bin", "--seq-len", "31", "--batch-size", "4"],
+                                   ["--layout", "packed", "--batch-size", "2", "--seq-len", "256"]], ids=["shards", "packed"])
+def test_first_step_loss_equals_the_oracle_forward(dev, tmp_path, extra):
+    """The first step of the harness (initial weights, first batch of the loader / the synthetic batch) against the
+    oracle's forward on the same weights and batch: 1e-3 relative, the bf16 loss bar."""
+    import glob
+    from collections import OrderedDict
+
+    from maltos_amd.data import PretrainingDataLoader, TokenShardDataset
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+    from oracle import llama as ol
+
+    out = tmp_path / "summary.json"
+    assert tp.main(["--model", "llama-tiny", "--steps", "2", "--warmup", "0", "--out", str(out), *extra]) == 0
+    summary = json.loads(out.read_text())
+    # the harness's initial weights: torch.manual_seed(seed), default construction, matrices redrawn N(0, 0.02)
+    torch.manual_seed(1234)
+    model = LlamaForCausalLM(LlamaConfig(**tp.MODELS["llama-tiny"]))
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() >= 2:
+                p.normal_(0.0, 0.02)
+    params = OrderedDict((n, p.detach().to(torch.bfloat16).float().to(dev)) for n, p in model.named_parameters())
+    if "--shards" in extra:
+        loader = PretrainingDataLoader(TokenShardDataset(sorted(glob.glob("tests/golden/tokens_0000*.bin"))), seq_len=31,
+                                       micro_batch_size=4, seed=1234)
+        batch = {k: v.to(dev) for k, v in loader.next_batch().items()}
+    else:
+        batch = tp.make_synthetic_batch(batch_size=2, seq_len=256, vocab_size=8192, layout="packed", seed=1234, device=dev)
+    cfg = ol.OracleLlamaConfig(**tp.MODELS["llama-tiny"])
+    want = ol.forward(params, cfg, batch[tp.INPUT_IDS_KEY], batch[tp.LABELS_KEY], position_ids=batch.get(tp.POSITION_IDS_KEY),
+                      sequence_ids=batch.get(tp.SEQUENCE_IDS_KEY))
+    assert abs(summary["loss_first"] - float(want)) <= 1e-3 * float(want), (summary["loss_first"], float(want))
