@@ -23,12 +23,19 @@ import time
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E peak
-# HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script scaled
-# by the same counters over the --calibrate-traffic kernel (summary: profiles/attn_cfg2_hbm_traffic.md).  Counters
-# cannot be read from inside the timed run, so the figures are carried here and refreshed with the profile.
-MEASURED_HBM_TRAFFIC_BYTES = {"attn_fwd": 679.1e6, "attn_bwd_dkdv": 1965.8e6, "attn_bwd_dq_ds": 1425.9e6,
-                              # the recomputing dQ kernel and the dK/dV kernel without the dS hand-over (the default backward)
-                              "attn_bwd_dq": 651.3e6, "attn_bwd_dkdv_recompute": 885.8e6}
+PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+
+
+def measured_hbm_traffic():
+    """HBM bytes per launch of each attention kernel on the headline workload: profiles/attn_cfg2_hbm_traffic.json, which
+    `python -m maltos_amd.profile_summary traffic` writes from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
+    WRITE_SIZE, each scaled by the same counter over the --calibrate-traffic kernel).  Counters cannot be read from
+    inside the timed run; a missing file gives null figures."""
+    try:
+        with open(os.path.join(PROFILES, "attn_cfg2_hbm_traffic.json")) as f:
+            return {k: v["hbm_bytes_per_launch"] for k, v in json.load(f)["kernels"].items()}
+    except (OSError, KeyError, ValueError):
+        return {}
 
 
 def parse_args():
@@ -37,7 +44,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-extra", action="store_true", help="only the headline attention workload")
-    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline legs")
+    ap.add_argument("--only", default=None, help="run only this leg of `extra` (for profiling one part of the run)")
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="only launch the streaming kernel of known size (mlts_scale over 1 GiB of fp32: 1 GiB read, "
                          "1 GiB written per launch) that the FETCH_SIZE / WRITE_SIZE counters are scaled against")
@@ -68,8 +76,8 @@ def timed(torch, fn, steps, warmup):
         gc.enable()
 
 
-def bench_attention(torch, ops, _lib, dev, steps, warmup):
-    B, H, S, D = 4, 16, 4096, 128
+def bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(4, 16, 4096, 128)):
+    B, H, S, D = shape
     q, k, v, do = attention_inputs(torch, dev, B, H, S, D)
     fwd_flops = 4.0 * B * H * S * S * D / 2.0
     flops = {"fwd": fwd_flops, "bwd": 2.5 * fwd_flops}
@@ -128,6 +136,114 @@ def bench_attention_handover(torch, ops, _lib, dev, steps, warmup):
         ops.set_backward_ds_handover_limit(previous)
     return {"value": (flops["fwd"] + flops["bwd"]) / sec / 1e12, "unit": "TFLOP/s", "ms_per_step": sec * 1e3,
             "kernels": kernels, "workspace_bytes": 2 * 4 * 16 * 4096 * 4096}
+
+
+def bench_attention_d64(torch, ops, _lib, dev, steps, warmup):
+    """The attention of the LLaMA-50M step alone: B=8, H=8, S=2048, head_dim 64, causal, bf16."""
+    sec, flops, kernels, _ = bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(8, 8, 2048, 64))
+    value = (flops["fwd"] + flops["bwd"]) / sec / 1e12
+    return {"workload": "causal self-attention fwd+bwd, B=8 H=8 S=2048 D=64, bf16", "value": value, "unit": "TFLOP/s",
+            "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS, "ms_per_step": sec * 1e3, "kernels": kernels}
+
+
+def packed_rows(torch, B, S, gen):
+    """Documents of uniform length in [64, 2048] until the row is full, the last one cut (configuration 3); returns
+    positions, sequence ids and sum over documents of L^2 / 2."""
+    pos = torch.zeros(B, S, dtype=torch.long)
+    seq = torch.zeros(B, S, dtype=torch.long)
+    work = 0
+    for b in range(B):
+        i = d = 0
+        while i < S:
+            L = min(int(torch.randint(64, 2049, (1,), generator=gen)), S - i)
+            pos[b, i:i + L] = torch.arange(L)
+            seq[b, i:i + L] = d
+            work += L * L / 2.0
+            i, d = i + L, d + 1
+    return pos, seq, work
+
+
+def bench_cfg3_packed_gqa(torch, ops, _lib, dev, steps, warmup):
+    """Configuration 3: packed documents, grouped-query attention (32 query heads on 8 KV heads), forward + backward;
+    TFLOP/s on the score elements the drawn documents actually have (sum of L^2 / 2 per head)."""
+    B, S, Hq, Hkv, D = 2, 8192, 32, 8, 128
+    gen = torch.Generator().manual_seed(1234)
+    pos, seq, work = packed_rows(torch, B, S, gen)
+    q = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    k = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    v = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    do = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    ids = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+
+    def step():
+        o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, **ids)
+        ops.attention_backward(do, q, k, v, o, lse, mask_mode=ops.MASK_DOC, **ids)
+
+    sec = timed(torch, step, steps, warmup)
+    flops = 3.5 * 4.0 * Hq * D * work
+    return {"workload": "packed documents (lengths uniform in [64, 2048]) causal attention fwd+bwd, B=2 S=8192 Hq=32 Hkv=8 D=128, bf16",
+            "score_elements_per_head": work, "flops_per_step": flops, "ms_per_step": sec * 1e3,
+            "value": flops / sec / 1e12, "unit": "TFLOP/s", "frac_of_mfma_peak": flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+
+def bench_cfg4_ring_rank(torch, dev, steps, warmup, rank=1):
+    """Configuration 4: one rank's share of zigzag ring attention at CP=4 over 32768 tokens (local Q of 8192 tokens against
+    the four KV chunks, all resident; block kernels + fp32 LSE merges forward, then the backward with the global O / LSE).
+    4 balanced blocks = 134,217,728 score elements per head: 3.848 TFLOP per rank."""
+    from maltos_amd.ring_attention import zigzag_ring_attention
+    from maltos_amd.ring_layout import expected_zigzag_ring_positions
+
+    W, H, S_loc, D = 4, 16, 8192, 128
+    gen = torch.Generator().manual_seed(1234)
+    gq, gk, gv, gdo = (torch.randn(1, H, W * S_loc, D, generator=gen).bfloat16().to(dev) for _ in range(4))
+    pos = [expected_zigzag_ring_positions(S_loc, rank=r, world_size=W, device=dev) for r in range(W)]
+    q = gq.index_select(2, pos[rank]).requires_grad_(True)
+    do = gdo.index_select(2, pos[rank])
+    chunks = [(gk.index_select(2, p_).requires_grad_(True), gv.index_select(2, p_).requires_grad_(True)) for p_ in pos]
+    del gq, gk, gv, gdo
+
+    def step():
+        out = zigzag_ring_attention(q, chunks, rank=rank, world_size=W)
+        out.backward(do)
+        q.grad = None
+        for kc, vc in chunks:
+            kc.grad = vc.grad = None
+
+    sec = timed(torch, step, steps, warmup)
+    flops = 3.5 * 4.0 * H * D * (W * S_loc * S_loc / 2.0)
+    return {"workload": f"zigzag ring attention fwd+bwd, rank {rank} of CP=4 over 32768 tokens, local Q 8192, H=16 D=128, bf16, merges included",
+            "flops_per_step": flops, "ms_per_step": sec * 1e3, "value": flops / sec / 1e12, "unit": "TFLOP/s",
+            "frac_of_mfma_peak": flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}
+
+
+def parity_cfg2(torch, ops, dev):
+    """Largest absolute and relative-to-largest-value differences of O, LSE, dQ, dK, dV on the headline inputs (first
+    batch element, all heads) against the library routine the configuration names: PyTorch SDPA, math backend, fp32,
+    differentiated by autograd."""
+    import torch.nn.functional as F
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    B, H, S, D = 4, 16, 4096, 128
+    q, k, v, do = (t[:1] for t in attention_inputs(torch, dev, B, H, S, D))
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o, lse = ops.attention(qg, kg, vg, mask_mode=ops.MASK_CAUSAL, return_lse=True)
+    o.backward(do)
+    qf, kf, vf = (t.float().requires_grad_(True) for t in (q, k, v))
+    with sdpa_kernel(SDPBackend.MATH):
+        want = F.scaled_dot_product_attention(qf, kf, vf, is_causal=True)
+    want.backward(do.float())
+    out = {}
+    for name, got, ref in (("O", o, want), ("dQ", qg.grad, qf.grad), ("dK", kg.grad, kf.grad), ("dV", vg.grad, vf.grad)):
+        err = (got.float() - ref.detach()).abs().max().item()
+        out[name] = {"max_abs": err, "rel": err / ref.detach().abs().max().item()}
+    scores = (qf.detach() @ kf.detach().transpose(-1, -2)) * D ** -0.5
+    scores.masked_fill_(~torch.ones(S, S, dtype=torch.bool, device=dev).tril(), float("-inf"))
+    want_lse = torch.logsumexp(scores, dim=-1)
+    err = (lse - want_lse).abs().max().item()
+    out["LSE"] = {"max_abs": err, "rel": err / want_lse.abs().max().item()}
+    out["reference"] = "torch SDPA math backend in fp32 on the bf16-rounded inputs, batch element 0 of configuration 2"
+    out["bound"] = "2e-2 max-abs (O, dQ, dK, dV), 2e-3 (LSE)"
+    return out
 
 
 def bench_adamw(torch, ops, _lib, dev, steps, warmup):
@@ -312,6 +428,82 @@ def cpu_baseline(torch):
                       f"(1/32 of the workload, same S and D), {reps} repeats, {sec * 1e3:.0f} ms each"}
 
 
+def llama_cfg_inputs(torch, cfg_dict, batch, seq, seed=1234):
+    """Initial weights (matrices N(0, 0.02), norm weights 1, in named_parameters order) and token ids of a LLaMA
+    configuration, drawn from one CPU generator."""
+    from collections import OrderedDict
+
+    from oracle import llama as ol
+
+    cfg = ol.OracleLlamaConfig(**cfg_dict)
+    gen = torch.Generator().manual_seed(seed)
+    params = OrderedDict()
+    for name, shape in ol.param_shapes(cfg).items():
+        params[name] = torch.randn(shape, generator=gen) * 0.02 if len(shape) >= 2 else torch.ones(shape)
+    ids = torch.randint(0, cfg.vocab_size, (batch, seq + 1), generator=gen)
+    return cfg, params, ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
+
+
+CFG1 = dict(vocab_size=8192, hidden_size=256, intermediate_size=688, num_hidden_layers=4, num_attention_heads=4,
+            max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=10000.0)
+CFG5 = dict(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8, num_attention_heads=8,
+            max_position_embeddings=2048, rms_norm_eps=1e-5, rope_theta=10000.0)
+
+
+def cpu_baseline_llama(torch, dev, which):
+    """One full train step (forward, backward, clip for configuration 5, stock AdamW on fp32 masters) of the CPU oracle
+    on the host cores at full size, next to the same first step through the HIP path from identical weights and
+    tokens: time, tokens/s and the parity of loss and gradient norm."""
+    from maltos_amd.grad_clip import clip_grad_norm_
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+    from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
+    from oracle import llama as ol
+
+    cfg_dict, batch, seq, dtype, max_norm = ((CFG1, 8, 256, torch.float32, None) if which == "cfg1"
+                                             else (CFG5, 8, 2048, torch.bfloat16, 1.0))
+    cfg, params, inp, lab = llama_cfg_inputs(torch, cfg_dict, batch, seq)
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    rounded = {n: p.to(dtype).float() for n, p in params.items()}   # the oracle evaluates the rounded network in fp32
+    timed_steps = 2 if which == "cfg1" else 1
+    ol.train_step(rounded, cfg, inp, lab, max_norm=max_norm) if which == "cfg1" else None   # warm-up (small case only)
+    t0 = time.perf_counter()
+    for _ in range(timed_steps):
+        want_loss, want_norm, _ = ol.train_step(rounded, cfg, inp, lab, max_norm=max_norm)
+    cpu_sec = (time.perf_counter() - t0) / timed_steps
+    model = LlamaForCausalLM(LlamaConfig(**cfg_dict)).to(dev)
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            p.copy_(params[n])
+    model = model.to(dtype)
+    adam = lambda ps: FusedAdamW(ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    opt = MasterWeightsOptimizer(model.parameters(), optimizer_factory=adam) if dtype != torch.float32 else adam(model.parameters())
+    data = {"input_ids": inp.to(dev), "labels": lab.to(dev)}
+    first = {}
+
+    def step():
+        loss = model(data)
+        loss.backward()
+        norm = clip_grad_norm_(opt, max_norm if max_norm is not None else float("inf"))   # inf: the norm only
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        first.setdefault("loss", float(loss.detach()))
+        first.setdefault("norm", float(norm))
+
+    step()
+    gpu_sec = timed(torch, step, 10, 3)
+    tokens = batch * seq
+    return {"workload": f"{'tiny LLaMA fp32 (configuration 1)' if which == 'cfg1' else 'LLaMA-50M bf16 (configuration 5)'} full train step, "
+                        f"batch {batch} x {seq}",
+            "cpu": {"ms": cpu_sec * 1e3, "tokens_per_sec": tokens / cpu_sec, "cores": torch.get_num_threads(), "kind": "port",
+                    "sample": f"oracle.llama.train_step (fp32 PyTorch restatement, stock AdamW) at full size, {timed_steps} timed step(s)"
+                              + (", 1 warm-up" if which == "cfg1" else ", no warm-up")},
+            "gpu": {"ms": gpu_sec * 1e3, "tokens_per_sec": tokens / gpu_sec},
+            "parity": {"loss": {"hip": first["loss"], "oracle": want_loss, "rel": abs(first["loss"] - want_loss) / abs(want_loss)},
+                       "grad_norm": {"hip": first["norm"], "oracle": want_norm, "rel": abs(first["norm"] - want_norm) / abs(want_norm)},
+                       "bound": "1e-4 relative (fp32)" if which == "cfg1" else "1e-3 relative (bf16)"}}
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -356,8 +548,7 @@ def main() -> int:
                    "flops_per_step": total_flops, "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS},
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": dom["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": dom["tflops"] / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(
-                         "attn_bwd_dkdv_recompute" if dominant == "attn_bwd_dkdv" and "attn_bwd_dq" in kernels else dominant),
+                     "traffic": measured_hbm_traffic().get(dominant),
                      "kernel_ms": dom["ms"], "algorithmic_flops_per_launch": kernel_flops[dominant]},
         "kernels": kernels,
     }
@@ -366,6 +557,8 @@ def main() -> int:
 
         def leg(name, fn):
             # a secondary figure that cannot be produced is reported as such; the headline line is still printed
+            if args.only is not None and name != args.only:
+                return
             try:
                 extra[name] = fn()
             except Exception as exc:  # noqa: BLE001
@@ -373,12 +566,19 @@ def main() -> int:
                 torch.cuda.synchronize()
 
         half = max(5, args.steps // 2)
+        leg("parity_cfg2", lambda: parity_cfg2(torch, ops, dev))
         leg("attn_ds_handover_backward", lambda: bench_attention_handover(torch, ops, _lib, dev, args.steps, args.warmup))
+        leg("attn_d64", lambda: bench_attention_d64(torch, ops, _lib, dev, args.steps, args.warmup))
+        leg("cfg3_packed_gqa", lambda: bench_cfg3_packed_gqa(torch, ops, _lib, dev, half, args.warmup))
+        leg("cfg4_ring_rank", lambda: bench_cfg4_ring_rank(torch, dev, half, 3))
         leg("adamw_flat_fp32", lambda: bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup))
         leg("hbm_kernels", lambda: bench_hbm_kernels(torch, ops, _lib, dev))
         leg("llama50m_train_step", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup)))
         leg("llama50m_train_step_graph", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), graph=True))
         leg("llama50m_train_step_zero1_layout", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), zero1=True))
+        if not args.skip_cpu:
+            leg("cfg1_tiny_llama_step_vs_cpu", lambda: cpu_baseline_llama(torch, dev, "cfg1"))
+            leg("cfg5_llama50m_step_vs_cpu", lambda: cpu_baseline_llama(torch, dev, "cfg5"))
         result["extra"] = extra
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
