@@ -18,7 +18,8 @@ import torch
 from maltos_amd import ops
 from maltos_amd.attention_backend import causal_attention
 from maltos_amd.flash_utils import (flash_attn_dense, flash_attn_dense_backward, flash_attn_dense_with_lse,
-                                    flash_attn_varlen)
+                                    flash_attn_varlen, flash_attn_varlen_prefix, flash_attn_varlen_prefix_backward,
+                                    flash_attn_varlen_prefix_with_lse)
 from maltos_amd.llama import HipAttentionCore
 from maltos_amd.ring_attention import HipRingAttentionCore, packed_ring_attention, zigzag_ring_attention
 from maltos_amd.ring_layout import expected_zigzag_ring_positions
@@ -345,6 +346,95 @@ def test_packed_ring_reference_scenario_fp32(dev, known_answers):
             dv_sum.index_add_(2, idx[src], v.grad.cpu())
     assert torch.allclose(dk_sum, gk.grad, atol=2e-5)
     assert torch.allclose(dv_sum, gv.grad, atol=2e-5)
+
+
+def test_prefix_function_set_drives_the_packed_ring_schedule(dev, known_answers):
+    """The reference's packed-document ring (runtime/layers/functional.py:823-1009) written against the provider
+    functions it calls, flash_attn_varlen_prefix_with_lse / _backward with allow_empty_kv=True, on the scenario of
+    tests/sequence_ids_attention_mask.py:366-434: per step one block forward merged into the running state, in the
+    backward one block backward from the merged out / LSE; the result is global document-masked attention."""
+    spec = known_answers["packed_ring"]
+    w, s_loc, total = spec["world_size"], spec["local_seq_len"], spec["local_seq_len"] * spec["world_size"]
+    mk = lambda seed: torch.randn((spec["batch"], spec["heads"], total, spec["head_dim"]), generator=torch.Generator().manual_seed(seed))
+    all_q, all_k, all_v = (mk(spec["seeds"][n]) for n in "qkv")
+    all_pos = torch.tensor(spec["positions"]).view(1, total)
+    all_seq = torch.tensor(spec["sequence_ids"]).view(1, total)
+    idx = [expected_zigzag_ring_positions(s_loc, rank=r, world_size=w, device=torch.device("cpu")) for r in range(w)]
+    gq, gk, gv = (t.clone().requires_grad_(True) for t in (all_q, all_k, all_v))
+    gout, glse = oa.attention_with_lse(gq, gk, gv, oa.doc_mask(all_pos, all_pos, all_seq, all_seq))
+    dout_all = torch.randn(gout.shape, generator=torch.Generator().manual_seed(5))
+    gout.backward(dout_all)
+    pc = [all_pos.index_select(1, i).to(dev) for i in idx]
+    sc = [all_seq.index_select(1, i).to(dev) for i in idx]
+    kc = [all_k.index_select(2, i).to(dev) for i in idx]
+    vc = [all_v.index_select(2, i).to(dev) for i in idx]
+    dk_sum, dv_sum = torch.zeros_like(all_k), torch.zeros_like(all_v)
+    for rank in range(w):
+        q = all_q.index_select(2, idx[rank]).to(dev)
+        running_out = torch.zeros(q.shape, dtype=torch.float32, device=dev)
+        running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=dev)
+        for step in range(w):
+            src = (rank - step) % w
+            block = flash_attn_varlen_prefix_with_lse(q, kc[src], vc[src], q_positions=pc[rank], k_positions=pc[src],
+                                                      q_sequence_ids=sc[rank], k_sequence_ids=sc[src], allow_empty_kv=True)
+            ops.attention_merge_(running_out, running_lse, block.out, block.lse)
+        assert torch.allclose(running_out.cpu(), gout.detach().index_select(2, idx[rank]), atol=spec["forward_atol"])
+        fin = torch.isfinite(glse.index_select(2, idx[rank]))
+        assert torch.equal(torch.isfinite(running_lse.cpu()), fin)
+        dout = dout_all.index_select(2, idx[rank]).to(dev)
+        dq = torch.zeros_like(q)
+        for step in range(w):
+            src = (rank - step) % w
+            bdq, bdk, bdv = flash_attn_varlen_prefix_backward(dout, q, kc[src], vc[src], running_out, running_lse, q_positions=pc[rank],
+                                                              k_positions=pc[src], q_sequence_ids=sc[rank], k_sequence_ids=sc[src],
+                                                              allow_empty_kv=True)
+            dq += bdq
+            dk_sum.index_add_(2, idx[src], bdk.cpu())
+            dv_sum.index_add_(2, idx[src], bdv.cpu())
+        assert torch.allclose(dq.cpu(), gq.grad.index_select(2, idx[rank]), atol=2e-5)
+    assert torch.allclose(dk_sum, gk.grad, atol=2e-5) and torch.allclose(dv_sum, gv.grad, atol=2e-5)
+
+
+def test_prefix_functions_empty_prefix_and_router_form(dev):
+    """A chunk of queries at positions 0, 1, 6, 7 against keys at positions 2..5 (the reference's own empty-prefix vector,
+    tests/sequence_ids_attention_mask.py:142-164): queries 0 and 1 see nothing.  allow_empty_kv=True gives zeros and
+    LSE = -inf there (runtime/layers/flash_utils.py:810-819), the strict forms raise like the reference's packer; the
+    differentiable form agrees with the oracle where every query has keys, GQA and bf16 included."""
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(1, 2, 4, 64, generator=g).to(dev) for _ in range(3))
+    q_pos, k_pos = torch.tensor([[0, 1, 6, 7]], device=dev), torch.tensor([[2, 3, 4, 5]], device=dev)
+    block = flash_attn_varlen_prefix_with_lse(q, k, v, q_positions=q_pos, k_positions=k_pos, allow_empty_kv=True)
+    assert torch.equal(block.out[:, :, :2].cpu(), torch.zeros(1, 2, 2, 64)) and torch.isneginf(block.lse[:, :, :2]).all()
+    want, want_lse = oa.attention_with_lse(q[:, :, 2:].cpu(), k.cpu(), v.cpu(), None)
+    check(block.out[:, :, 2:], want, torch.float32, "prefix block")
+    check(block.lse[:, :, 2:], want_lse, torch.float32, "prefix block LSE")
+    dq, dk, dv = flash_attn_varlen_prefix_backward(torch.ones_like(q), q, k, v, block.out, block.lse, q_positions=q_pos, k_positions=k_pos,
+                                                   allow_empty_kv=True)
+    assert torch.equal(dq[:, :, :2].cpu(), torch.zeros(1, 2, 2, 64)) and torch.isfinite(dk).all() and torch.isfinite(dv).all()
+    with pytest.raises(ValueError, match="without any matching key/value prefix"):
+        flash_attn_varlen_prefix_with_lse(q, k, v, q_positions=q_pos, k_positions=k_pos)
+    with pytest.raises(ValueError, match="without any matching key/value prefix"):
+        flash_attn_varlen_prefix(q, k, v, q_positions=q_pos, k_positions=k_pos)
+    with pytest.raises(ValueError, match="k_positions shape must match"):
+        flash_attn_varlen_prefix(q, k, v, q_positions=q_pos, k_positions=k_pos[:, :3])
+
+    gen = torch.Generator().manual_seed(9)
+    B, Hq, Hkv, Sq, Sk, D = 2, 4, 2, 192, 320, 128
+    pos, seq = make_docs(B, Sk, gen, 90, pad_tail=11)
+    take = torch.arange(Sk - Sq, Sk)  # the queries are the last Sq tokens of the gathered keys
+    qb, kb, vb, dob = bshd(B, Hq, Sq, D, gen, torch.bfloat16), bshd(B, Hkv, Sk, D, gen, torch.bfloat16), bshd(B, Hkv, Sk, D, gen, torch.bfloat16), bshd(B, Hq, Sq, D, gen, torch.bfloat16)
+    qpos, qseq = pos[:, take], seq[:, take]
+    qf, kf, vf = (t.detach().float().clone().requires_grad_(True) for t in (qb, kb, vb))
+    want_o, _ = oa.attention_with_lse(qf, kf, vf, oa.doc_mask(qpos, pos, qseq, seq))
+    want_o.backward(dob.float())
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (qb, kb, vb))
+    out = flash_attn_varlen_prefix(qd, kd, vd, q_positions=qpos.to(dev), k_positions=pos.to(dev), q_sequence_ids=qseq.to(dev),
+                                   k_sequence_ids=seq.to(dev))
+    out.backward(dob.to(dev))
+    check(out, want_o.detach(), torch.bfloat16, "prefix O")
+    check(qd.grad, qf.grad, torch.bfloat16, "prefix dQ")
+    check(kd.grad, kf.grad, torch.bfloat16, "prefix dK")
+    check(vd.grad, vf.grad, torch.bfloat16, "prefix dV")
 
 
 @pytest.mark.parametrize("D", [64, 128])

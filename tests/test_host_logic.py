@@ -14,7 +14,7 @@ from maltos_amd import _lib, ops
 from maltos_amd.attention_backend import (ATTENTION_BACKEND_CHOICES, AttentionBackend, causal_attention,
                                           validate_attention_backend)
 from maltos_amd.attn_masking_utils import build_example_causal_mask, canonical_position_ids, canonical_sequence_ids
-from maltos_amd.flash_utils import varlen_qkv_metadata
+from maltos_amd.flash_utils import varlen_prefix_metadata, varlen_qkv_metadata
 from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
 from maltos_amd.ring_attention import zigzag_ring_schedule
 from maltos_amd.ring_layout import expected_zigzag_ring_positions, has_zigzag_ring_layout
@@ -170,6 +170,68 @@ def test_varlen_metadata_known_answers(known_answers):
     assert again is not meta and again.cu_seqlens.tolist() == e["cu_seqlens"]
     empty = varlen_qkv_metadata(torch.full((2, 3), -1))
     assert empty.cu_seqlens.tolist() == [0] and empty.max_seqlen == 0
+
+
+def _prefix_layout_by_hand(q_pos, k_pos, q_seq, k_seq, allow_empty):
+    """Token-by-token walk of the rule stated in the reference (runtime/layers/flash_utils.py:627-690), for small cases."""
+    q_idx, k_idx, q_len, k_len = [], [], [], []
+    B, Sq = q_pos.shape
+    Sk = k_pos.size(1)
+    for b in range(B):
+        toks = [i for i in range(Sq) if int(q_seq[b, i]) != -1]
+        runs, cur = [], []
+        for i in toks:
+            if cur and (int(q_seq[b, i]) != int(q_seq[b, cur[-1]]) or int(q_pos[b, i]) != int(q_pos[b, cur[-1]]) + 1):
+                runs.append(cur)
+                cur = []
+            cur.append(i)
+        if cur:
+            runs.append(cur)
+        for run in runs:
+            sid, end = int(q_seq[b, run[0]]), int(q_pos[b, run[-1]])
+            keys = [j for j in range(Sk) if int(k_seq[b, j]) == sid and int(k_seq[b, j]) != -1 and int(k_pos[b, j]) <= end]
+            if not keys:
+                assert allow_empty
+                continue
+            q_idx += [b * Sq + i for i in run]
+            k_idx += [b * Sk + j for j in keys]
+            q_len.append(len(run))
+            k_len.append(len(keys))
+    return q_idx, k_idx, q_len, k_len
+
+
+def test_varlen_prefix_metadata_known_answers(known_answers):
+    for case in known_answers["varlen_prefix_pack"]["cases"]:
+        t = lambda name: None if case[name] is None else torch.tensor(case[name])
+        meta = varlen_prefix_metadata(q_positions=t("q_positions"), k_positions=t("k_positions"), q_sequence_ids=t("q_sequence_ids"),
+                                      k_sequence_ids=t("k_sequence_ids"), allow_empty_kv=case["allow_empty_kv"])
+        assert meta.cu_seqlens_q.tolist() == case["cu_seqlens_q"] and meta.cu_seqlens_q.dtype == torch.int32
+        assert meta.cu_seqlens_k.tolist() == case["cu_seqlens_k"] and meta.cu_seqlens_k.dtype == torch.int32
+        assert (meta.max_seqlen_q, meta.max_seqlen_k) == (case["max_seqlen_q"], case["max_seqlen_k"])
+        assert meta.q_indices.tolist() == case["q_indices"] and meta.k_indices.tolist() == case["k_indices"]
+    empty_case = known_answers["varlen_prefix_pack"]["cases"][1]
+    with pytest.raises(ValueError, match="without any matching key/value prefix"):
+        varlen_prefix_metadata(q_positions=torch.tensor(empty_case["q_positions"]), k_positions=torch.tensor(empty_case["k_positions"]))
+    none = varlen_prefix_metadata(q_positions=torch.zeros(2, 3, dtype=torch.long), k_positions=torch.zeros(2, 3, dtype=torch.long),
+                                  q_sequence_ids=torch.full((2, 3), -1), k_sequence_ids=torch.zeros(2, 3, dtype=torch.long))
+    assert none.cu_seqlens_q.tolist() == [0] and none.max_seqlen_q == 0 and none.q_indices.numel() == 0
+
+
+def test_varlen_prefix_metadata_against_token_walk():
+    gen = torch.Generator().manual_seed(11)
+    for trial in range(20):
+        B, Sq, Sk = 2, 13, 17
+        # shuffled chunks of a few documents with padding: positions and ids drawn so that runs break in every way
+        q_seq = torch.randint(-1, 3, (B, Sq), generator=gen)
+        k_seq = torch.randint(-1, 3, (B, Sk), generator=gen)
+        q_pos = torch.cumsum(torch.randint(0, 3, (B, Sq), generator=gen), 1) % 7
+        k_pos = torch.randint(0, 7, (B, Sk), generator=gen)
+        want = _prefix_layout_by_hand(q_pos, k_pos, q_seq, k_seq, True)
+        meta = varlen_prefix_metadata(q_positions=q_pos, k_positions=k_pos, q_sequence_ids=q_seq, k_sequence_ids=k_seq, allow_empty_kv=True)
+        assert meta.q_indices.tolist() == want[0] and meta.k_indices.tolist() == want[1], trial
+        assert (meta.cu_seqlens_q[1:] - meta.cu_seqlens_q[:-1]).tolist() == want[2]
+        assert (meta.cu_seqlens_k[1:] - meta.cu_seqlens_k[:-1]).tolist() == want[3]
+        assert meta.max_seqlen_q == max(want[2], default=0) and meta.max_seqlen_k == max(want[3], default=0)
 
 
 def test_optimizer_plumbing_on_host():
