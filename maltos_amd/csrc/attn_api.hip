@@ -7,7 +7,7 @@
 
 int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st);                        // attn_fwd_dma.hip
 int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq);                             // attn_bwd_split.hip
-int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st);    // attn_bwd_split.hip
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, bool lse2_ready, hipStream_t st);    // attn_bwd_split.hip
 int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
 int64_t mlts_attn_bwd_ds_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t Sk);                              // attn_bwd_dq_ds.hip
 int mlts_attn_bwd_dq_bf16_ds(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_ds.hip
@@ -176,18 +176,28 @@ int64_t bwd_min_workspace(const mlts_attn_shape* s) {
   return stats_bytes(s) + delta + lse2;
 }
 
-// dK/dV kernel, then the dQ kernel: from the handed-over dS when ds_ws is set, by recomputation otherwise
-int attn_bwd_bf16(AttnBwdParams bp, int D, int mode, void* lse2_ws, void* ds_ws, hipStream_t st) {
+// Default: the recomputing dQ kernel first, which also writes the row statistics (delta, lse2) into the workspace, then
+// the dK/dV kernel that reads them.  With a dS hand-over (ds_ws): statistics passes, dK/dV kernel, dQ from its dS.
+int attn_bwd_bf16(AttnBwdParams bp, int D, int mode, float* delta_ws, void* lse2_ws, void* ds_ws, bool stats_in_dq,
+                  hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + 127) / 128;
   if (ds_ws) {
     bp.ds_ws = ds_ws;
     bp.ds_nkb = (p.Sk + 31) / 32;
     bp.ds_nqt = (p.Sq + 63) / 64;
+    int rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, lse2_ws, false, st);
+    if (rc != MLTS_OK) return rc;
+    return mlts_attn_bwd_dq_bf16_ds(bp, D, mode, st);
   }
-  int rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, lse2_ws, st);
+  if (stats_in_dq) {
+    bp.delta_out = delta_ws;
+    bp.lse2_out = static_cast<float*>(lse2_ws);
+  }
+  int rc = mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
   if (rc != MLTS_OK) return rc;
-  return ds_ws ? mlts_attn_bwd_dq_bf16_ds(bp, D, mode, st) : mlts_attn_bwd_dq_bf16_tr(bp, D, mode, st);
+  bp.delta_out = bp.lse2_out = nullptr;
+  return mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, lse2_ws, stats_in_dq, st);
 }
 
 int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
@@ -219,6 +229,7 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
   bp.nkt = 0;
   bp.ds_ws = nullptr;
   bp.ds_nkb = bp.ds_nqt = 0;
+  bp.delta_out = bp.lse2_out = nullptr;
   if (uses_mfma(s)) {
     MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
                      mlts_aligned16(dq) && mlts_aligned16(dk) && mlts_aligned16(dv),
@@ -229,16 +240,21 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
                  "%s: strides must keep rows 16-byte aligned", who);
     MLTS_REQUIRE(do_stride[2] < kMaxRowStride, "%s: the sequence stride of dout must be below 2^24 elements", who);
   }
-  if (s->Sq > 0) {
+  void* lse2_ws = ws;
+  void* ds_ws = nullptr;
+  if (uses_mfma(s)) {
+    ws += mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);
+    const int64_t ds_bytes = ds_handover_bytes(s, accumulate_f32);
+    if (ds_bytes > 0 && workspace_bytes >= need + ds_bytes) ds_ws = ws;
+  }
+  // the recomputing dQ kernel forms delta itself from 16-byte chunks of the O rows
+  const bool stats_in_dq = uses_mfma(s) && !ds_ws && s->Sk > 0 && mlts_aligned16(o) && strides_aligned(s->o_stride, 2);
+  if (s->Sq > 0 && !stats_in_dq) {
     int rc = mlts_attn_delta(dout, do_stride, o, s->o_stride, delta, s->B, s->Hq, s->Sq, s->D, s->dtype, st);
     if (rc != MLTS_OK) return rc;
   }
   if (!uses_mfma(s)) return mlts_attn_generic_bwd(bp, s->D, s->dtype, s->mask_mode, st);
-  void* lse2_ws = ws;
-  ws += mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);
-  const int64_t ds_bytes = ds_handover_bytes(s, accumulate_f32);
-  void* ds_ws = ds_bytes > 0 && workspace_bytes >= need + ds_bytes ? ws : nullptr;
-  return attn_bwd_bf16(bp, s->D, s->mask_mode, lse2_ws, ds_ws, st);
+  return attn_bwd_bf16(bp, s->D, s->mask_mode, delta, lse2_ws, ds_ws, stats_in_dq, st);
 }
 
 // ---- scratch of the entry point that allocates nothing --------------------------------------------------------

@@ -30,7 +30,8 @@ struct DqCfg {
   static constexpr int TILE_BYTES = BN * RB;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
   static constexpr int PRO_BYTES = 2 * BM * RB;        // the prologue passes the Q and dO tiles through LDS
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES > PRO_BYTES ? STAGES * STAGE_BYTES : PRO_BYTES;
+  static constexpr int DELTA_OFF = STAGES * STAGE_BYTES > PRO_BYTES ? STAGES * STAGE_BYTES : PRO_BYTES;  // delta[BM], fp32
+  static constexpr int LDS_BYTES = DELTA_OFF + BM * 4;
   static constexpr int NLD = BN * CPR / THREADS;       // 16-byte chunks per thread and tile (2 or 1)
 };
 
@@ -118,8 +119,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   // layout) and handed to the wavefronts through LDS: a fragment load straight from global memory touches 32 rows per
   // instruction and was measured at ~90 cycles per instruction, 8 us for the workgroup.  Rows past the end repeat
   // the last query (their lse2 is +inf, so they contribute nothing and are never stored).
+  //
+  // With bp.delta_out set, this kernel also produces the row statistics of the whole backward: it fetches the O rows
+  // next to the dO rows, forms delta = rowsum(dO * O) from the chunks it holds (a row's CPR chunks sit in CPR
+  // neighbouring lanes) and writes delta and lse2 for its rows; the dK/dV kernel, launched afterwards, reads them.
   constexpr int NPRO = BM * CPR / THREADS;
+  const bool fold_stats = bp.delta_out != nullptr;
+  const int64_t stat_off = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow;
   v4i32 pro_q[NPRO], pro_d[NPRO];
+  float pro_dot[NPRO];
 #pragma unroll
   for (int n = 0; n < NPRO; ++n) {
     const int c = tid + n * THREADS;
@@ -129,11 +137,35 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     pro_q[n] = *reinterpret_cast<const v4i32*>(Q + r * p.qs[2] + col);
     pro_d[n] = *reinterpret_cast<const v4i32*>(dO + r * bp.dos[2] + col);
   }
+  if (fold_stats) {
+    const bf16_t* O = static_cast<const bf16_t*>(p.o) + b * p.os[0] + hq * p.os[1];
+    v4i32 pro_o[NPRO];
+#pragma unroll
+    for (int n = 0; n < NPRO; ++n) {
+      const int c = tid + n * THREADS;
+      const int row = c / CPR;
+      const int col = ((c % CPR) ^ swz<D>(row & 15)) * 8;
+      const int64_t r = min(q0 + row, p.Sq - 1);
+      pro_o[n] = *reinterpret_cast<const v4i32*>(O + r * p.os[2] + col);
+    }
+#pragma unroll
+    for (int n = 0; n < NPRO; ++n) {
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {  // two bf16 per 32-bit word: low half = even element
+        acc += __builtin_bit_cast(float, pro_d[n][i] << 16) * __builtin_bit_cast(float, pro_o[n][i] << 16);
+        acc += __builtin_bit_cast(float, pro_d[n][i] & static_cast<int>(0xffff0000u)) *
+               __builtin_bit_cast(float, pro_o[n][i] & static_cast<int>(0xffff0000u));
+      }
+#pragma unroll
+      for (int m = CPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m, 64);
+      pro_dot[n] = acc;
+    }
+  }
   float lse_raw = -INFINITY, delta = 0.f;
   if (qrow < p.Sq) {
-    const int64_t off = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq + qrow;
-    lse_raw = p.lse[off];
-    delta = bp.delta[off];
+    lse_raw = p.lse[stat_off];
+    if (!fold_stats) delta = bp.delta[stat_off];
   }
   int qpos = 0, qseq = -1;
   int4 wq_stats = make_int4(0, -1, 0, -1);
@@ -242,6 +274,11 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       lds_write_b128<0>(wbase + n * (THREADS * 16), pro_q[n]);
       lds_write_b128<0>(wbase + BM * RB + n * (THREADS * 16), pro_d[n]);
     }
+    if (fold_stats && tid % CPR == 0) {
+      float* sdelta = reinterpret_cast<float*>(smem + C::DELTA_OFF);
+#pragma unroll
+      for (int n = 0; n < NPRO; ++n) sdelta[tid / CPR + n * (THREADS / CPR)] = pro_dot[n];
+    }
     drain_and_barrier();
     v4i32 fq[KS], fd[KS];
 #pragma unroll
@@ -258,10 +295,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       qf[ks] = as_frag(fq[ks]);
       ndof[ks] = as_frag(fd[ks]);
     }
+    if (fold_stats) delta = reinterpret_cast<const float*>(smem + C::DELTA_OFF)[wave * 32 + l32];
     drain_and_barrier();  // the K/V tiles may overwrite the Q and dO tiles from here on
   }
   // +inf makes exp2(s - lse2) = 0 for rows that saw no key or lie past Sq
   const float lse2 = lse_raw == -INFINITY ? INFINITY : lse_raw * kLog2e;
+  if (fold_stats) {
+    if (qrow < p.Sq && hh == 0) {
+      bp.delta_out[stat_off] = delta;
+      bp.lse2_out[stat_off] = lse2;
+    }
+    if (bid == 0 && tid == 0) bp.lse2_out[static_cast<int64_t>(p.B) * p.Hq * p.Sq] = INFINITY;
+  }
 
   f32x16 dqacc[DB];  // -dQ^T / scale: register e <-> head-dim 32 db + 8 (e/4) + 4 hh + e%4, lane -> query row
 #pragma unroll

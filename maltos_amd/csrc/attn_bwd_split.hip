@@ -765,11 +765,13 @@ int launch_mode(const AttnBwdParams& bp, int mode, const float* lse2, hipStream_
 int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq) { return (((B * Hq * Sq + 1) * 4 + 255) / 256) * 256; }
 
 // head_dim 64 or 128, 16-byte aligned rows (checked by the caller); workspace holds B*Hq*Sq + 1 floats.
-int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, hipStream_t st) {
+// lse2_ready: the workspace already holds lse2 (written by the dQ kernel that ran before).
+int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, bool lse2_ready, hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + BKV - 1) / BKV;
   float* lse2 = static_cast<float*>(workspace);
   const int64_t n = static_cast<int64_t>(p.B) * p.Hq * p.Sq;
-  hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 256) / 256)), dim3(256), 0, st, p.lse, lse2, n);
+  if (!lse2_ready)
+    hipLaunchKernelGGL(lse2_kernel, dim3(static_cast<unsigned>((n + 256) / 256)), dim3(256), 0, st, p.lse, lse2, n);
   return D == 128 ? launch_mode<128>(bp, mode, lse2, st) : launch_mode<64>(bp, mode, lse2, st);
 }

@@ -48,6 +48,11 @@ struct AttnBwdParams {
   // of the tile (the A-operand order of the dK product).  Blocks that no query can see are not written.
   void* ds_ws;
   int ds_nkb, ds_nqt;
+  // Optional outputs of the recomputing dQ kernel, which then runs first and takes the place of the separate row
+  // statistics passes: delta_out[B, Hq, Sq] = rowsum(dO * O) (the kernel ignores `delta` and reads `a.o`), and
+  // lse2_out[B * Hq * Sq + 1] = lse * log2(e) with +inf for rows that saw no key and in the last entry.
+  float* delta_out;
+  float* lse2_out;
 };
 
 // whether block (32-key block kb, 64-query tile qt) of the dS hand-over is written (MLTS_MASK_NONE / MLTS_MASK_CAUSAL)

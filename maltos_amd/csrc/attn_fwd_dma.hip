@@ -120,16 +120,6 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
   bf16_t* O = static_cast<bf16_t*>(p.o) + b * p.os[0] + hq * p.os[1];
 
-  bf16x8 qf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    if (qrow < p.Sq) {
-      qf[ks] = *reinterpret_cast<const bf16x8*>(Q + static_cast<int64_t>(qrow) * p.qs[2] + ks * 16 + hh * 8);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) qf[ks][i] = static_cast<bf16_t>(0.f);
-    }
-  }
   int qpos = 0, qseq = -1;
   int4 wq_stats = make_int4(0, -1, 0, -1);
   int4 bq_stats[BM / 64];
@@ -254,8 +244,37 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     --inflight;
     issue_next();
   };
-  issue_next();
-  issue_next();
+  // ---- Q: this wavefront's 32 rows travel like a K tile (whole rows by LDS-DMA, same row layout and swizzle) into the
+  // ring stages that the first two tiles do not use, and come back as B-operand fragments with one ds_read_b128 each.
+  // (A fragment gathered straight from global memory touches 32 cache lines per instruction: eight such loads per
+  // wavefront took most of the time before the first tile.)  Rows past the end repeat the last row; they are never
+  // stored.  Every wavefront reads its fragments before its first sync(), whose barrier therefore also says that
+  // stages 2 and 3 are free for tiles 2 and 3. ----
+  bf16x8 qf[KS];
+  {
+    constexpr int QP = 32 * RB / 1024;  // 1 KiB pieces of this wavefront's rows
+    unsigned char* qbase = smem + 2 * STAGE_BYTES + wave * (32 * RB);
+#pragma unroll
+    for (int n = 0; n < QP; ++n) {
+      const int row = n * (64 / CPR) + lane / CPR;
+      const int col = ((lane % CPR) ^ swz<D>(row & 15)) * 8;
+      const int r = min(wq0 + row, p.Sq - 1);
+      __builtin_amdgcn_global_load_lds(MLTS_GLB(Q + static_cast<int64_t>(r) * p.qs[2] + col), MLTS_LDS(qbase + n * 1024), 16, 0, 0);
+    }
+    issue_next();
+    issue_next();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    v4i32 qraw[KS];
+    const uint32_t qa = lds0 + 2 * STAGE_BYTES + wave * (32 * RB);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qraw[ks] = lds_read_b128<0>(qa + koff[ks]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+v"(qraw[ks]));  // the fragments are used only behind the wait above
+      qf[ks] = as_frag(qraw[ks]);
+    }
+  }
 
   f32x16 sacc[2];
   bf16x8 pf[4];
