@@ -173,6 +173,15 @@ int mlts_rope(const void* x, const int64_t x_stride[3], void* y, const int64_t y
               int32_t B, int32_t H, int32_t S, int32_t D, int32_t dtype, int32_t inverse,
               mlts_stream_t stream);
 
+/* The two rotations of one attention layer, q = rotary(q) and k = rotary(k) (models/llama.py:143-144), in one launch:
+ * operand a is [B, Ha, S, D], operand b [B, Hb, S, D]; everything else as mlts_rope, whose results it equals bit for
+ * bit.  Each operand must hold fewer than 2^31 16-byte vectors. */
+int mlts_rope_pair(const void* xa, const int64_t xa_stride[3], void* ya, const int64_t ya_stride[3], int32_t Ha,
+                   const void* xb, const int64_t xb_stride[3], void* yb, const int64_t yb_stride[3], int32_t Hb,
+                   const void* cos_tab, const void* sin_tab, int32_t max_pos, const int32_t* positions,
+                   int32_t position_offset, int32_t B, int32_t S, int32_t D, int32_t dtype, int32_t inverse,
+                   mlts_stream_t stream);
+
 /* h = round(silu(gate)) * up (models/llama.py:205-206); n = number of elements, contiguous. */
 int mlts_swiglu_fwd(const void* gate, const void* up, void* h, int64_t n, int32_t dtype, mlts_stream_t stream);
 int mlts_swiglu_bwd(const void* dh, const void* gate, const void* up, void* dgate, void* dup, int64_t n,

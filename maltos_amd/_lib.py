@@ -91,6 +91,11 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
         [_P, _I64P, _P, _I64P, _P, _P, C.c_int32, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
          C.c_int32, C.c_int32, _P],
     ),
+    "mlts_rope_pair": (
+        C.c_int,
+        [_P, _I64P, _P, _I64P, C.c_int32, _P, _I64P, _P, _I64P, C.c_int32, _P, _P, C.c_int32, _P, C.c_int32, C.c_int32,
+         C.c_int32, C.c_int32, C.c_int32, C.c_int32, _P],
+    ),
     "mlts_swiglu_fwd": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, _P]),
     "mlts_swiglu_bwd": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int32, _P]),
     "mlts_ce_workspace_bytes": (C.c_int64, [C.c_int64]),

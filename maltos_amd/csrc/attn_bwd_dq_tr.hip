@@ -31,7 +31,9 @@ struct DqCfg {
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
   static constexpr int PRO_BYTES = 2 * BM * RB;        // the prologue passes the Q and dO tiles through LDS
   static constexpr int DELTA_OFF = STAGES * STAGE_BYTES > PRO_BYTES ? STAGES * STAGE_BYTES : PRO_BYTES;  // delta[BM], fp32
-  static constexpr int LDS_BYTES = DELTA_OFF + BM * 4;
+  static constexpr int META_OFF = DELTA_OFF + BM * 4;  // document masks: per stage k_pos[64] then k_seq[64], int32
+  static constexpr int META_BYTES = 2 * BN * 4;
+  static constexpr int LDS_BYTES = META_OFF + STAGES * META_BYTES;
   static constexpr int NLD = BN * CPR / THREADS;       // 16-byte chunks per thread and tile (2 or 1)
 };
 
@@ -191,17 +193,12 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     j_end = lim < 0 ? 0 : min(nkt, lim / BN + 1);
   }
   const int wave_last_q = min(wq0 + 31, p.Sq - 1);
-  auto block_needs = [&](int j) -> bool {
-    if (MODE != MLTS_MASK_DOC) return true;
-    const int4 ks4 = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
-    bool need = false;
-#pragma unroll
-    for (int w = 0; w < BM / 64; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
-    return need;
-  };
+  // needed tiles in increasing order (document masks: 64 tiles of statistics per step)
+  DocTileScan scan;
+  const int4* k_stats_row = MODE == MLTS_MASK_DOC ? p.k_stats + static_cast<int64_t>(b) * p.nk_stats : nullptr;
   auto next_tile = [&](int j) -> int {
-    while (j < j_end && !block_needs(j)) ++j;
-    return j;
+    if (MODE != MLTS_MASK_DOC) return j < j_end ? j : j_end;
+    return doc_scan_next<BM / 64, true>(scan, j, j_end, p.nk_stats, k_stats_row, bq_stats, wq_stats, lane);
   };
 
   // ---- tile loader: 64 bytes per thread, chunks t and t + 512 of the K tile and of the V tile (chunk c = row c/16,
@@ -219,8 +216,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     ld_voff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n]) * 2;
   }
   v4i32 stg_k[NLD], stg_v[NLD];
+  int stg_m = 0;  // document masks: threads 0..127 carry the tile's key positions (64) and sequence ids (64)
   auto stage_load = [&](int j) {
     const int kv0 = j * BN;
+    if (MODE == MLTS_MASK_DOC && tid < 2 * BN) {
+      const int32_t* src = (tid < BN ? p.k_pos : p.k_seq) + static_cast<int64_t>(b) * p.Sk;
+      stg_m = src[min(kv0 + (tid & (BN - 1)), p.Sk - 1)];
+    }
     const bf16_t* Kt = K + static_cast<int64_t>(kv0) * p.ks[2];
     const bf16_t* Vt = V + static_cast<int64_t>(kv0) * p.vs[2];
     const int last = p.Sk - 1 - kv0;  // rows past the end repeat the last key; their scores are masked
@@ -245,6 +247,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       lds_write_b128<THREADS * 16>(a, stg_k[NLD - 1]);
       lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_v[NLD - 1]);
     }
+    if (MODE == MLTS_MASK_DOC && tid < 2 * BN)
+      asm volatile("ds_write_b32 %0, %1" ::"v"(lds0 + C::META_OFF + stage * C::META_BYTES + tid * 4), "v"(stg_m));
   };
 
   const int j0 = next_tile(0);
@@ -339,24 +343,22 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     f32x16 s, dp;
     // masked tiles only (a wave-uniform branch around VALU work, no matrix instruction inside): hidden scores -> -inf
     auto apply_mask = [&](const int kb) {
+      // document masks: positions and sequence ids of the keys come from the stage's copy, four keys at a time (the
+      // registers of a whole block's worth are not to be had at this point of the tile)
+      const uint32_t ma = lds0 + C::META_OFF + (so / STAGE_BYTES) * C::META_BYTES + (kb * 32 + hh * 4) * 4;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
-        int kp[4], ksq[4];
+        v4i32 kp[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [0] positions, [1] sequence ids of keys kb * 32 + g * 8 + hh * 4 .. + 3
         if (MODE == MLTS_MASK_DOC) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int kj = kbase + r;
-            const bool ok = kj < p.Sk;
-            kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
-            ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
-          }
+          kp[0] = g == 0 ? lds_read_b128<0>(ma) : g == 1 ? lds_read_b128<32>(ma) : g == 2 ? lds_read_b128<64>(ma) : lds_read_b128<96>(ma);
+          kp[1] = g == 0 ? lds_read_b128<BN * 4>(ma) : g == 1 ? lds_read_b128<BN * 4 + 32>(ma) : g == 2 ? lds_read_b128<BN * 4 + 64>(ma) : lds_read_b128<BN * 4 + 96>(ma);
+          wait_lgkm<0>(kp);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
           bool vis = kb * 32 + g * 8 + r <= klim_t;
-          if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+          if (MODE == MLTS_MASK_DOC) vis = vis && (kp[0][r] <= qpos) && (kp[1][r] == qseq) && (qseq >= 0);
           if (!vis) s[g * 4 + r] = -INFINITY;
         }
       }
@@ -437,6 +439,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     if (j < j_end) stage_store(0);
     int stage = 0;
     while (j < j_end) {
+      const int doc_cls = MODE == MLTS_MASK_DOC ? doc_scan_class(scan, j) : TILE_FULL;  // before the scan moves on
       const int jn = next_tile(j + 1);
       drain_and_barrier();
       if (jn < j_end) stage_load(jn);
@@ -447,7 +450,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
         if (kv0 > wave_last_q + p.causal_off) cls = TILE_SKIP;
         else if (kv0 + BN - 1 > wq0 + p.causal_off) cls = TILE_MASKED;
       } else if (MODE == MLTS_MASK_DOC) {
-        cls = classify_doc_tile(wq_stats, p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j]);
+        cls = doc_cls;
       }
       if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;  // ragged last tile: key < Sk
       if (wq0 >= p.Sq) cls = TILE_SKIP;

@@ -36,8 +36,8 @@ struct SplitCfg {
   static constexpr int RB = D * 2;                   // bytes per tile row
   static constexpr int CPR = RB / 16;                // 16-byte chunks per row
   static constexpr int TILE_BYTES = BQ * RB;
-  static constexpr int STAT_OFF = 2 * TILE_BYTES;    // lse2[64] then delta[64], fp32
-  static constexpr int STAGE_BYTES = STAT_OFF + 2 * BQ * 4;
+  static constexpr int STAT_OFF = 2 * TILE_BYTES;    // lse2[64], delta[64] (fp32), then q_pos[64], q_seq[64] (int32, document masks)
+  static constexpr int STAGE_BYTES = STAT_OFF + 4 * BQ * 4;
   static constexpr int PBUF_OFF = STAGES * STAGE_BYTES;
   static constexpr int LDS_BYTES = PBUF_OFF + 2 * 4 * PBUF_BYTES;
   static constexpr int NLD = BQ * CPR / THREADS;     // 16-byte chunks per thread and tile (2 or 1)
@@ -81,6 +81,10 @@ __device__ __forceinline__ void lds_write_b128(uint32_t addr, v4i32 x) {
 template <int N>
 __device__ __forceinline__ void wait_lgkm(v4i32 (&x)[4]) {
   asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[2]) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x[0]), "+v"(x[1]) : "n"(N));
 }
 template <int N>
 __device__ __forceinline__ void wait_lgkm(v4i32 (&x)[8]) {
@@ -174,19 +178,27 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     int qt, h;  // query tile relative to qt_begin, head within the GQA group
   };
   auto at_end = [&](const Pos& x) -> bool { return x.h >= group || span == 0; };
-  auto tile_needed = [&](const Pos& x) -> bool {
-    if (MODE != MLTS_MASK_DOC) return true;
-    const int4 qs4 = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt_begin + x.qt];
-    return classify_doc_tile(qs4, kstats[0]) != TILE_SKIP || classify_doc_tile(qs4, kstats[1]) != TILE_SKIP;
-  };
   auto step = [&](Pos& x) {
     if (++x.qt == span) {
       x.qt = 0;
       ++x.h;
     }
   };
+  // document masks: the needed query tiles (the same for every head of the group) are found 64 tiles of statistics
+  // at a time; scan positions are relative to qt_begin
+  DocTileScan scan;
+  const int4* q_stats_row = MODE == MLTS_MASK_DOC ? p.q_stats + static_cast<int64_t>(b) * p.nq_stats + qt_begin : nullptr;
   auto first_needed = [&](Pos x) -> Pos {  // x itself or the next position whose tile is needed
-    while (!at_end(x) && !tile_needed(x)) step(x);
+    if (MODE != MLTS_MASK_DOC) return x;
+    while (!at_end(x)) {
+      const int q = doc_scan_next<2, false>(scan, x.qt, span, span, q_stats_row, kstats, wk_stats, lane);
+      if (q < span) {
+        x.qt = q;
+        return x;
+      }
+      x.qt = 0;
+      ++x.h;
+    }
     return x;
   };
   auto classify = [&](const Pos& x) -> int {  // for this wavefront's 32 keys; identical in both roles of a key block
@@ -198,7 +210,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       if (wkv0 > last_q + p.causal_off) cls = TILE_SKIP;
       else if (wkv0 + 31 > q0 + p.causal_off) cls = TILE_MASKED;
     } else if (MODE == MLTS_MASK_DOC) {
-      cls = classify_doc_tile(p.q_stats[static_cast<int64_t>(b) * p.nq_stats + qt], wk_stats);
+      cls = doc_scan_class(scan, x.qt);
     }
     if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || q0 + BQ > p.Sq)) cls = TILE_MASKED;
     if (wkv0 >= p.Sk) cls = TILE_SKIP;
@@ -248,6 +260,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
       const int r = q0 + (tid & (BQ - 1));
       stg_s = tid < BQ ? lse2[r < p.Sq ? srow + r : lse2_inf] : bp.delta[srow + min(r, p.Sq - 1)];
+    } else if (MODE == MLTS_MASK_DOC && tid < 4 * BQ) {
+      // the tile's query positions and sequence ids (as raw bits), for the tiles whose mask is evaluated pair by pair;
+      // rows past the end are padding
+      const int r = q0 + (tid & (BQ - 1));
+      const int32_t* src = (tid < 3 * BQ ? p.q_pos : p.q_seq) + static_cast<int64_t>(b) * p.Sq;
+      const int v = r < p.Sq ? src[r] : (tid < 3 * BQ ? -0x7fffffff : -1);
+      stg_s = __builtin_bit_cast(float, v);
     }
   };
   const uint32_t stg_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem))) + tid * 16;
@@ -259,7 +278,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       lds_write_b128<THREADS * 16>(a, stg_q[NLD - 1]);
       lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_d[NLD - 1]);
     }
-    if (tid < 2 * BQ)
+    if (tid < (MODE == MLTS_MASK_DOC ? 4 : 2) * BQ)
       asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(lds0_ + stage * STAGE_BYTES + tid * 4), "v"(stg_s), "n"(STAT_OFF));
   };
 
@@ -348,18 +367,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       // hoisting all of them in front of the wave-uniform branch, where every tile would pay for them
       int causal_here = causal_t;
       asm volatile("" : "+v"(causal_here));
+      // document masks: positions and sequence ids of the queries come from the stage, four queries at a time
+      const uint32_t ma = sb + STAT_OFF + 2 * BQ * 4 + (qb * 32 + hh * 4) * 4;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int qrow = qb * 32 + g * 8 + hh * 4;
-        int qp4[4], qs4[4];
+        v4i32 qm[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [0] positions, [1] sequence ids of queries qb * 32 + g * 8 + hh * 4 .. + 3
         if (MODE == MLTS_MASK_DOC) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int qi = q0 + qrow + r;
-            const bool ok = qi < p.Sq;
-            qp4[r] = ok ? p.q_pos[static_cast<int64_t>(b) * p.Sq + qi] : -0x7fffffff;
-            qs4[r] = ok ? p.q_seq[static_cast<int64_t>(b) * p.Sq + qi] : -1;
-          }
+          qm[0] = g == 0 ? lds_read_b128<0>(ma) : g == 1 ? lds_read_b128<32>(ma) : g == 2 ? lds_read_b128<64>(ma) : lds_read_b128<96>(ma);
+          qm[1] = g == 0 ? lds_read_b128<BQ * 4>(ma) : g == 1 ? lds_read_b128<BQ * 4 + 32>(ma) : g == 2 ? lds_read_b128<BQ * 4 + 64>(ma) : lds_read_b128<BQ * 4 + 96>(ma);
+          wait_lgkm<0>(qm);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -367,8 +383,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
           if (MODE == MLTS_MASK_CAUSAL) {
             vis = causal_here <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
           } else {
-            const int qi = q0 + qrow + r;
-            vis = kj < p.Sk && qi < p.Sq && (kpos <= qp4[r]) && (kseq == qs4[r]) && (qs4[r] >= 0);
+            vis = kj < p.Sk && (kpos <= qm[0][r]) && (kseq == qm[1][r]) && (qm[1][r] >= 0);
           }
           if (!vis) s[g * 4 + r] = -INFINITY;
         }
@@ -641,13 +656,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     int prev_stage = 0;
     Pos prev_it = it;
     while (!at_end(it)) {
+      const int cls = classify(it);  // before the scan of the needed tiles moves on
       Pos itn = it;
       step(itn);
       itn = first_needed(itn);
       drain_and_barrier();
       if (!at_end(itn)) stage_load(itn);
       const int q0 = (qt_begin + it.qt) * BQ;
-      const int cls = classify(it);
       const int pbuf = (k & 1) * (4 * PBUF_BYTES);
       if (ROLE == 0) {
         // one instance of the tile body (with several, the register allocator keeps the accumulators twice); the

@@ -74,4 +74,59 @@ __device__ __forceinline__ int classify_doc_tile(const int4 qs, const int4 ks) {
   return TILE_MASKED;
 }
 
+// MLTS_MASK_DOC: which tiles of one batch row's tile statistics a workgroup needs and how one wavefront sees them,
+// evaluated 64 tiles at a time (lane i looks at tile base + i, the answers travel as wave-uniform 64-bit masks).
+// Walking the statistics one tile at a time costs a dependent global load per tile, needed or not, which is as long
+// as the work on a needed tile.
+struct DocTileScan {
+  unsigned long long need = 0, skip = 0, full = 0;  // bit i <-> tile base + i
+  int base = -64;                                   // no chunk loaded
+};
+
+// KEYS = true: the scanned tiles are key tiles, `grp` / `own` are query statistics (forward, dQ); false: the scanned
+// tiles are query tiles and `grp` / `own` key statistics (dK/dV).  need: some group of `grp` sees the tile; skip / full:
+// classification against `own`.
+template <int NG, bool KEYS>
+__device__ __forceinline__ void doc_scan_fill(DocTileScan& sc, int base, int n_tiles, const int4* __restrict__ row_stats,
+                                              const int4 (&grp)[NG], const int4 own, int lane) {
+  const int t = base + lane;
+  bool need = false, skip = true, full = false;
+  if (t < n_tiles) {
+    const int4 ts = row_stats[t];
+#pragma unroll
+    for (int w = 0; w < NG; ++w) need |= (KEYS ? classify_doc_tile(grp[w], ts) : classify_doc_tile(ts, grp[w])) != TILE_SKIP;
+    const int c = KEYS ? classify_doc_tile(own, ts) : classify_doc_tile(ts, own);
+    skip = c == TILE_SKIP;
+    full = c == TILE_FULL;
+  }
+  sc.need = __builtin_amdgcn_ballot_w64(need);
+  sc.skip = __builtin_amdgcn_ballot_w64(skip);
+  sc.full = __builtin_amdgcn_ballot_w64(full);
+  sc.base = base;
+}
+
+// first needed tile in [j, end), or end; n_tiles = number of statistics entries of the row
+template <int NG, bool KEYS>
+__device__ __forceinline__ int doc_scan_next(DocTileScan& sc, int j, int end, int n_tiles, const int4* __restrict__ row_stats,
+                                             const int4 (&grp)[NG], const int4 own, int lane) {
+  while (j < end) {
+    if (j < sc.base || j >= sc.base + 64) doc_scan_fill<NG, KEYS>(sc, j & ~63, n_tiles, row_stats, grp, own, lane);
+    const unsigned long long m = sc.need >> (j - sc.base);
+    if (m != 0) {
+      const int t = j + __builtin_ctzll(m);
+      return t < end ? t : end;
+    }
+    j = sc.base + 64;
+  }
+  return end;
+}
+
+// classification of tile j for the wavefront; j must lie in the chunk the scan holds (it does right after
+// doc_scan_next returned it)
+__device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
+  const int bit = j - sc.base;
+  if ((sc.skip >> bit) & 1ull) return TILE_SKIP;
+  return ((sc.full >> bit) & 1ull) ? TILE_FULL : TILE_MASKED;
+}
+
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);

@@ -29,7 +29,9 @@ struct FwdCfg {
   static constexpr int CPR = RB / 16;                  // 16-byte chunks per row
   static constexpr int TILE_BYTES = BN * RB;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+  static constexpr int META_OFF = STAGES * STAGE_BYTES;     // document masks: per stage k_pos[64] then k_seq[64], int32
+  static constexpr int META_BYTES = 2 * BN * 4;
+  static constexpr int LDS_BYTES = META_OFF + STAGES * META_BYTES;
   static constexpr int PPW = TILE_BYTES / (WAVES * 1024);  // 1 KiB pieces of each tile per wavefront (2 or 1)
   static constexpr int LOADS_PER_TILE = 2 * PPW;           // DMA instructions per wavefront per stage
 };
@@ -96,7 +98,9 @@ template <int D, int MODE>
 __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams p) {
   using C = FwdCfg<D>;
   constexpr int KS = C::KS, DB = C::DB, RB = C::RB, CPR = C::CPR, TILE_BYTES = C::TILE_BYTES, STAGE_BYTES = C::STAGE_BYTES,
-                PPW = C::PPW, LOADS_PER_TILE = C::LOADS_PER_TILE;
+                PPW = C::PPW, META_OFF = C::META_OFF, META_BYTES = C::META_BYTES;
+  // DMA instructions per wavefront and tile; with document masks one more: 16 of the tile's 128 position / sequence ids
+  constexpr int LOADS_PER_TILE = C::LOADS_PER_TILE + (MODE == MLTS_MASK_DOC ? 1 : 0);
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: everything derived from it stays scalar
@@ -144,17 +148,12 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     j_end = lim < 0 ? 0 : min(nkt, lim / BN + 1);
   }
   const int wave_last_q = min(wq0 + 31, p.Sq - 1);
-  auto block_needs = [&](int j) -> bool {
-    if (MODE != MLTS_MASK_DOC) return true;
-    const int4 ks4 = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
-    bool need = false;
-#pragma unroll
-    for (int w = 0; w < BM / 64; ++w) need |= classify_doc_tile(bq_stats[w], ks4) != TILE_SKIP;
-    return need;
-  };
-  auto next_tile = [&](int j) -> int {
-    while (j < j_end && !block_needs(j)) ++j;
-    return j;
+  // needed tiles in increasing order: one cursor for the loader (two tiles ahead), one for the consumer
+  DocTileScan scan_load, scan_use;
+  const int4* k_stats_row = MODE == MLTS_MASK_DOC ? p.k_stats + static_cast<int64_t>(b) * p.nk_stats : nullptr;
+  auto next_tile = [&](DocTileScan& sc, int j) -> int {
+    if (MODE != MLTS_MASK_DOC) return j < j_end ? j : j_end;
+    return doc_scan_next<BM / 64, true>(sc, j, j_end, p.nk_stats, k_stats_row, bq_stats, wq_stats, lane);
   };
 
   // ---- DMA loader: this wavefront moves PPW 1 KiB pieces of the K tile and of the V tile; piece n holds rows
@@ -176,6 +175,15 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   auto issue_tile = [&](int j, int stage) {
     const int kv0 = j * BN;
     unsigned char* sbase = smem + stage * STAGE_BYTES + wave * PPW * 1024;
+    if (MODE == MLTS_MASK_DOC) {
+      // the tile's key positions and sequence ids, for the tiles that need the mask evaluated pair by pair: wavefront w
+      // moves entries 16 w .. 16 w + 15 of (k_pos[64], k_seq[64]) with its first 16 lanes
+      if (lane < 16) {
+        const int e = wave * 16 + lane;
+        const int32_t* src = (e < BN ? p.k_pos : p.k_seq) + static_cast<int64_t>(b) * p.Sk + min(kv0 + (e & (BN - 1)), p.Sk - 1);
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(src), MLTS_LDS(smem + META_OFF + stage * META_BYTES + wave * 64), 4, 0, 0);
+      }
+    }
     if (kv0 + BN <= p.Sk) {
       const unsigned char* kt = Kb + static_cast<int64_t>(kv0) * p.ks[2] * 2;
       const unsigned char* vt = Vb + static_cast<int64_t>(kv0) * p.vs[2] * 2;
@@ -229,12 +237,12 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   // wavefronts finished it two syncs ago, the late ones read its V before their QK(k - 1), i.e. before this sync.
   const bool late = wave >= WAVES / 2;
   int inflight = 0, istage = 0;
-  int ji = next_tile(0);
+  int ji = next_tile(scan_load, 0);
   auto issue_next = [&]() {
     if (ji < j_end) {
       issue_tile(ji, istage);
       istage = (istage + 1) & (STAGES - 1);
-      ji = next_tile(ji + 1);
+      ji = next_tile(scan_load, ji + 1);
       ++inflight;
     }
   };
@@ -331,11 +339,12 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       }
   };
 
-  int j = next_tile(0);
+  int j = next_tile(scan_use, 0);
   int stage = 0;
   if (late && j < j_end) sync();
   while (j < j_end) {
-    const int jn = next_tile(j + 1);
+    const int doc_cls = MODE == MLTS_MASK_DOC ? doc_scan_class(scan_use, j) : TILE_FULL;  // before the scan moves on
+    const int jn = next_tile(scan_use, j + 1);
     if (!late) sync();
     __builtin_amdgcn_s_setprio(1);  // the matrix block of this wavefront goes ahead of the other wavefront's softmax
     if (pv_pending) pv_phase();
@@ -346,7 +355,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       if (kv0 > wave_last_q + p.causal_off) cls = TILE_SKIP;
       else if (kv0 + BN - 1 > wq0 + p.causal_off) cls = TILE_MASKED;
     } else if (MODE == MLTS_MASK_DOC) {
-      cls = classify_doc_tile(wq_stats, p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j]);
+      cls = doc_cls;
     }
     if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;
     if (wq0 >= p.Sq) cls = TILE_SKIP;
@@ -403,25 +412,31 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       if (cls == TILE_MASKED) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
+          // document masks: positions and sequence ids of this key block's 16 keys per lane half, read from the stage's
+          // copy in one go (groups g = 0..3: keys kb * 32 + g * 8 + hh * 4 .. + 3)
+          v4i32 kp[4], ksq[4];
+          if (MODE == MLTS_MASK_DOC) {
+            const uint32_t ma = lds0 + META_OFF + stage * META_BYTES + (kb * 32 + hh * 4) * 4;
+            kp[0] = lds_read_b128<0>(ma);
+            kp[1] = lds_read_b128<32>(ma);
+            kp[2] = lds_read_b128<64>(ma);
+            kp[3] = lds_read_b128<96>(ma);
+            ksq[0] = lds_read_b128<BN * 4>(ma);
+            ksq[1] = lds_read_b128<BN * 4 + 32>(ma);
+            ksq[2] = lds_read_b128<BN * 4 + 64>(ma);
+            ksq[3] = lds_read_b128<BN * 4 + 96>(ma);
+            wait_lgkm<0>(kp[0], kp[1], kp[2], kp[3]);
+            wait_lgkm<0>(ksq[0], ksq[1], ksq[2], ksq[3]);
+          }
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
-            int kp[4], ksq[4];
-            if (MODE == MLTS_MASK_DOC) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                const int kj = kbase + r;
-                const bool ok = kj < p.Sk;
-                kp[r] = ok ? p.k_pos[static_cast<int64_t>(b) * p.Sk + kj] : 0x7fffffff;
-                ksq[r] = ok ? p.k_seq[static_cast<int64_t>(b) * p.Sk + kj] : -2;
-              }
-            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int kj = kbase + r;
               bool vis = kj < p.Sk;
               if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
-              if (MODE == MLTS_MASK_DOC) vis = vis && (kp[r] <= qpos) && (ksq[r] == qseq) && (qseq >= 0);
+              if (MODE == MLTS_MASK_DOC) vis = vis && (kp[g][r] <= qpos) && (ksq[g][r] == qseq) && (qseq >= 0);
               if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
             }
           }

@@ -219,15 +219,14 @@ int rmsnorm_bwd_blocks(int64_t rows) {
 // IDX is the type the flat element index is taken apart in: 32-bit whenever the tensor has fewer than 2^31 vectors
 // (three 64-bit divisions per lane cost several hundred instructions, more than the rotation itself).
 template <typename T, bool INVERSE, typename IDX>
-__global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
-                                                        T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
-                                                        const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
-                                                        int max_pos, const int32_t* __restrict__ positions,
-                                                        int position_offset, int B, int H, int S, int D) {
+__device__ __forceinline__ void rope_rows(const int64_t idx64, const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
+                                          T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
+                                          const T* __restrict__ cos_tab, const T* __restrict__ sin_tab, int max_pos,
+                                          const int32_t* __restrict__ positions, int position_offset, int B, int H, int S,
+                                          int D) {
   constexpr int N = Vec16<T>::N;
   const int vec_per_row = D / N;
   const int64_t total = static_cast<int64_t>(B) * S * H * vec_per_row;
-  const int64_t idx64 = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (idx64 >= total) return;
   // order (b, s, h, vec): neighbouring lanes touch neighbouring memory for [B, S, H, D] storage
   const IDX idx = static_cast<IDX>(idx64);
@@ -264,6 +263,36 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x,
     o.set(2 * j + 1, oo);
   }
   *reinterpret_cast<Vec16<T>*>(yp) = o;
+}
+
+template <typename T, bool INVERSE, typename IDX>
+__global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
+                                                        T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
+                                                        const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
+                                                        int max_pos, const int32_t* __restrict__ positions,
+                                                        int position_offset, int B, int H, int S, int D) {
+  rope_rows<T, INVERSE, IDX>(static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x, x, xsb, xsh, xss, y, ysb, ysh, yss,
+                             cos_tab, sin_tab, max_pos, positions, position_offset, B, H, S, D);
+}
+
+// Two tensors of one layer (the query and the key projections) in one launch: blocks [0, first_blocks) rotate the
+// first, the rest the second.  Same arithmetic as rope_kernel; a launch of this size costs more than it computes.
+struct RopeOperand {
+  const void* x;
+  void* y;
+  int64_t xs[3], ys[3];
+  int H;
+};
+template <typename T, bool INVERSE>
+__global__ __launch_bounds__(kThreads) void rope_pair_kernel(const RopeOperand a, const RopeOperand b, unsigned first_blocks,
+                                                             const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
+                                                             int max_pos, const int32_t* __restrict__ positions,
+                                                             int position_offset, int B, int S, int D) {
+  const bool second = blockIdx.x >= first_blocks;
+  const RopeOperand& t = second ? b : a;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x - (second ? first_blocks : 0u)) * kThreads + threadIdx.x;
+  rope_rows<T, INVERSE, uint32_t>(idx, static_cast<const T*>(t.x), t.xs[0], t.xs[1], t.xs[2], static_cast<T*>(t.y), t.ys[0],
+                                  t.ys[1], t.ys[2], cos_tab, sin_tab, max_pos, positions, position_offset, B, t.H, S, D);
 }
 
 // ============================== SwiGLU ===================================================
@@ -543,31 +572,80 @@ extern "C" int mlts_add_rmsnorm_bwd(const void* dy, const void* x, const void* w
                              hidden, dtype, stream);
 }
 
+// validation shared by mlts_rope and mlts_rope_pair
+static int rope_check(const char* who, const void* x, const int64_t* x_stride, const void* y, const int64_t* y_stride,
+                      const void* cos_tab, const void* sin_tab, int32_t max_pos, const int32_t* positions,
+                      int32_t position_offset, int32_t B, int32_t H, int32_t S, int32_t D, int32_t dtype) {
+  MLTS_REQUIRE(known_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  MLTS_REQUIRE(B >= 0 && H >= 0 && S >= 0 && D > 0, "%s: bad shape", who);
+  const int n = elem_per_vec(dtype);
+  const int esz = dtype == MLTS_BF16 ? 2 : 4;
+  MLTS_REQUIRE(D % n == 0, "%s: head_dim=%d must be a multiple of %d", who, D, n);
+  if (B == 0 || H == 0 || S == 0) return MLTS_OK;
+  MLTS_REQUIRE(x && y && cos_tab && sin_tab && x_stride && y_stride, "%s: null pointer", who);
+  MLTS_REQUIRE(max_pos > 0, "%s: max_pos must be positive", who);
+  MLTS_REQUIRE(positions != nullptr || (position_offset >= 0 && position_offset + S <= max_pos),
+               "%s: positions [%d, %d) exceed the table (%d rows)", who, position_offset, position_offset + S, max_pos);
+  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(y), "%s: x and y must be 16-byte aligned", who);
+  MLTS_REQUIRE((reinterpret_cast<uintptr_t>(cos_tab) & 7u) == 0 && (reinterpret_cast<uintptr_t>(sin_tab) & 7u) == 0,
+               "%s: the cos / sin tables must be 8-byte aligned", who);
+  for (int i = 0; i < 3; ++i)
+    MLTS_REQUIRE((x_stride[i] * esz) % 16 == 0 && (y_stride[i] * esz) % 16 == 0,
+                 "%s: strides must keep rows 16-byte aligned", who);
+  return MLTS_OK;
+}
+
 extern "C" int mlts_rope(const void* x, const int64_t x_stride[3], void* y, const int64_t y_stride[3],
                          const void* cos_tab, const void* sin_tab, int32_t max_pos, const int32_t* positions,
                          int32_t position_offset, int32_t B, int32_t H, int32_t S, int32_t D, int32_t dtype,
                          int32_t inverse, mlts_stream_t stream) {
-  MLTS_REQUIRE(known_dtype(dtype), "mlts_rope: unknown dtype %d", dtype);
-  MLTS_REQUIRE(B >= 0 && H >= 0 && S >= 0 && D > 0, "mlts_rope: bad shape");
-  const int n = elem_per_vec(dtype);
-  const int esz = dtype == MLTS_BF16 ? 2 : 4;
-  MLTS_REQUIRE(D % n == 0, "mlts_rope: head_dim=%d must be a multiple of %d", D, n);
+  if (int rc = rope_check("mlts_rope", x, x_stride, y, y_stride, cos_tab, sin_tab, max_pos, positions, position_offset, B,
+                          H, S, D, dtype); rc != MLTS_OK)
+    return rc;
   if (B == 0 || H == 0 || S == 0) return MLTS_OK;
-  MLTS_REQUIRE(x && y && cos_tab && sin_tab && x_stride && y_stride, "mlts_rope: null pointer");
-  MLTS_REQUIRE(max_pos > 0, "mlts_rope: max_pos must be positive");
-  MLTS_REQUIRE(positions != nullptr || (position_offset >= 0 && position_offset + S <= max_pos),
-               "mlts_rope: positions [%d, %d) exceed the table (%d rows)", position_offset, position_offset + S, max_pos);
-  MLTS_REQUIRE(mlts_aligned16(x) && mlts_aligned16(y), "mlts_rope: x and y must be 16-byte aligned");
-  MLTS_REQUIRE((reinterpret_cast<uintptr_t>(cos_tab) & 7u) == 0 && (reinterpret_cast<uintptr_t>(sin_tab) & 7u) == 0,
-               "mlts_rope: the cos / sin tables must be 8-byte aligned");
-  for (int i = 0; i < 3; ++i)
-    MLTS_REQUIRE((x_stride[i] * esz) % 16 == 0 && (y_stride[i] * esz) % 16 == 0,
-                 "mlts_rope: strides must keep rows 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == MLTS_BF16 ? rope_t<bf16_t>(x, x_stride, y, y_stride, cos_tab, sin_tab, max_pos, positions,
                                              position_offset, B, H, S, D, inverse, st)
                             : rope_t<float>(x, x_stride, y, y_stride, cos_tab, sin_tab, max_pos, positions,
                                             position_offset, B, H, S, D, inverse, st);
+}
+
+template <typename T>
+static int rope_pair_t(const RopeOperand& a, const RopeOperand& b, const void* ct, const void* sn, int max_pos,
+                       const int32_t* positions, int off, int B, int S, int D, int inverse, hipStream_t st) {
+  MltsKernelTimer timer("rope", st);
+  constexpr int N = Vec16<T>::N;
+  const int64_t per_head = static_cast<int64_t>(B) * S * (D / N);
+  const int64_t blocks_a = (per_head * a.H + kThreads - 1) / kThreads, blocks_b = (per_head * b.H + kThreads - 1) / kThreads;
+  if (inverse)
+    hipLaunchKernelGGL((rope_pair_kernel<T, true>), dim3((unsigned)(blocks_a + blocks_b)), dim3(kThreads), 0, st, a, b,
+                       (unsigned)blocks_a, static_cast<const T*>(ct), static_cast<const T*>(sn), max_pos, positions, off, B, S, D);
+  else
+    hipLaunchKernelGGL((rope_pair_kernel<T, false>), dim3((unsigned)(blocks_a + blocks_b)), dim3(kThreads), 0, st, a, b,
+                       (unsigned)blocks_a, static_cast<const T*>(ct), static_cast<const T*>(sn), max_pos, positions, off, B, S, D);
+  return mlts_check_launch("mlts_rope_pair");
+}
+
+extern "C" int mlts_rope_pair(const void* xa, const int64_t xa_stride[3], void* ya, const int64_t ya_stride[3], int32_t Ha,
+                              const void* xb, const int64_t xb_stride[3], void* yb, const int64_t yb_stride[3], int32_t Hb,
+                              const void* cos_tab, const void* sin_tab, int32_t max_pos, const int32_t* positions,
+                              int32_t position_offset, int32_t B, int32_t S, int32_t D, int32_t dtype, int32_t inverse,
+                              mlts_stream_t stream) {
+  if (int rc = rope_check("mlts_rope_pair", xa, xa_stride, ya, ya_stride, cos_tab, sin_tab, max_pos, positions,
+                          position_offset, B, Ha, S, D, dtype); rc != MLTS_OK)
+    return rc;
+  if (int rc = rope_check("mlts_rope_pair", xb, xb_stride, yb, yb_stride, cos_tab, sin_tab, max_pos, positions,
+                          position_offset, B, Hb, S, D, dtype); rc != MLTS_OK)
+    return rc;
+  if (B == 0 || S == 0 || (Ha == 0 && Hb == 0)) return MLTS_OK;
+  const int n = elem_per_vec(dtype);
+  MLTS_REQUIRE(static_cast<int64_t>(B) * S * (Ha > Hb ? Ha : Hb) * (D / n) < (1LL << 31),
+               "mlts_rope_pair: tensors of 2^31 or more 16-byte vectors go through mlts_rope");
+  RopeOperand a{xa, ya, {xa_stride[0], xa_stride[1], xa_stride[2]}, {ya_stride[0], ya_stride[1], ya_stride[2]}, Ha};
+  RopeOperand b{xb, yb, {xb_stride[0], xb_stride[1], xb_stride[2]}, {yb_stride[0], yb_stride[1], yb_stride[2]}, Hb};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == MLTS_BF16 ? rope_pair_t<bf16_t>(a, b, cos_tab, sin_tab, max_pos, positions, position_offset, B, S, D, inverse, st)
+                            : rope_pair_t<float>(a, b, cos_tab, sin_tab, max_pos, positions, position_offset, B, S, D, inverse, st);
 }
 
 extern "C" int mlts_swiglu_fwd(const void* gate, const void* up, void* h, int64_t n, int32_t dtype,

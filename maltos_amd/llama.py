@@ -194,8 +194,7 @@ class LlamaAttention(nn.Module):
         q = self.q_proj(x).view(batch, seq_len, self.num_heads, self.head_dim).transpose(1, 2)
         k = self.k_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
         v = self.v_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
-        q = ops.rope(q, cos, sin, positions=rope_pos, position_offset=position_offset)
-        k = ops.rope(k, cos, sin, positions=rope_pos, position_offset=position_offset)
+        q, k = ops.rope_pair(q, k, cos, sin, positions=rope_pos, position_offset=position_offset)
         if not getattr(self.attn_core, "preserves_native_gqa", False) and self.num_heads != self.num_kv_heads:
             rep = self.num_heads // self.num_kv_heads
             k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)

@@ -19,7 +19,7 @@ __all__ = [
     "MASK_NONE", "MASK_CAUSAL", "MASK_DOC",
     "attention", "attention_forward", "attention_backward", "attention_backward_accumulate", "attention_merge_",
     "set_backward_ds_handover_limit",
-    "rms_norm", "rope", "swiglu", "cross_entropy",
+    "rms_norm", "rope", "rope_pair", "swiglu", "cross_entropy",
     "adamw_step_", "sq_norm", "scale_", "grad_to_f32_",
 ]
 
@@ -312,6 +312,27 @@ def _rope(x, cos, sin, positions, position_offset, inverse):
     return y
 
 
+def _rope_pair(xa, xb, cos, sin, positions, position_offset, inverse):
+    """Both rotations of an attention layer (query and key projections) in one launch."""
+    _require_gpu(xa, xb, cos, sin, positions)
+    if xa.dim() != 4 or xb.dim() != 4 or xa.size(0) != xb.size(0) or xa.shape[2:] != xb.shape[2:] or xa.dtype != xb.dtype:
+        raise ValueError("rope_pair expects two [batch, heads, seq, head_dim] tensors that differ only in heads")
+    B, Ha, S, D = xa.shape
+    if cos.shape != sin.shape or cos.dim() != 2 or cos.size(1) * 2 != D:
+        raise ValueError(f"cos/sin tables must be [max_pos, {D // 2}], got {tuple(cos.shape)}")
+    if cos.dtype != xa.dtype or sin.dtype != xa.dtype:
+        raise ValueError("cos/sin tables must have the activation dtype (the reference casts them first)")
+    xa, xb = _dense_last(xa), _dense_last(xb)
+    ya, yb = torch.empty_like(xa), torch.empty_like(xb)
+    pos32 = None if positions is None else _ids32(positions, B, S, "position_ids")
+    cos, sin = cos.contiguous(), sin.contiguous()
+    _lib.check(_lib.lib().mlts_rope_pair(_p(xa), strides3(xa.stride()[:3]), _p(ya), strides3(ya.stride()[:3]), Ha,
+                                         _p(xb), strides3(xb.stride()[:3]), _p(yb), strides3(yb.stride()[:3]), xb.size(1),
+                                         _p(cos), _p(sin), cos.size(0), _p(pos32), int(position_offset), B, S, D,
+                                         _dtype_code(xa), int(bool(inverse)), _stream()))
+    return ya, yb
+
+
 def _swiglu_fwd(gate, up):
     _require_gpu(gate, up)
     if gate.shape != up.shape or gate.dtype != up.dtype:
@@ -363,6 +384,7 @@ _LIBRARY.define("rmsnorm_bwd(Tensor dy, Tensor x, Tensor w, Tensor rstd) -> (Ten
 _LIBRARY.define("add_rmsnorm_fwd(Tensor x, Tensor res, Tensor w, float eps) -> (Tensor, Tensor, Tensor)")
 _LIBRARY.define("add_rmsnorm_bwd(Tensor dy, Tensor dres, Tensor h, Tensor w, Tensor rstd) -> (Tensor, Tensor)")
 _LIBRARY.define("rope(Tensor x, Tensor cos, Tensor sin, Tensor? positions, int position_offset, bool inverse) -> Tensor")
+_LIBRARY.define("rope_pair(Tensor xa, Tensor xb, Tensor cos, Tensor sin, Tensor? positions, int position_offset, bool inverse) -> (Tensor, Tensor)")
 _LIBRARY.define("swiglu_fwd(Tensor gate, Tensor up) -> Tensor")
 _LIBRARY.define("swiglu_bwd(Tensor dh, Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _LIBRARY.define("ce_fwd_bwd(Tensor logits, Tensor labels, int ignore_index) -> (Tensor, Tensor, Tensor)")
@@ -385,7 +407,7 @@ def _cpu_refusal(name: str) -> None:
     _LIBRARY.impl(name, refuse, "CPU")
 
 
-for _name in ("attn_fwd", "attn_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "add_rmsnorm_fwd", "add_rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "ce_fwd_bwd",
+for _name in ("attn_fwd", "attn_bwd", "rmsnorm_fwd", "rmsnorm_bwd", "add_rmsnorm_fwd", "add_rmsnorm_bwd", "rope", "rope_pair", "swiglu_fwd", "swiglu_bwd", "ce_fwd_bwd",
               "scale_by_scalar", "scale_by_scalar_"):
     _cpu_refusal(_name)
 
@@ -406,6 +428,7 @@ _impl("rmsnorm_bwd")(_rmsnorm_bwd)
 _impl("add_rmsnorm_fwd")(_add_rmsnorm_fwd)
 _impl("add_rmsnorm_bwd")(_add_rmsnorm_bwd)
 _impl("rope")(_rope)
+_impl("rope_pair")(_rope_pair)
 _impl("swiglu_fwd")(_swiglu_fwd)
 _impl("swiglu_bwd")(_swiglu_bwd)
 _impl("ce_fwd_bwd")(_ce_fwd_bwd)
@@ -469,6 +492,11 @@ def _(dy, dres, h, w, rstd):
 @torch.library.register_fake("maltos::rope")
 def _(x, cos, sin, positions, position_offset, inverse):
     return torch.empty_like(x)
+
+
+@torch.library.register_fake("maltos::rope_pair")
+def _(xa, xb, cos, sin, positions, position_offset, inverse):
+    return torch.empty_like(xa), torch.empty_like(xb)
 
 
 @torch.library.register_fake("maltos::swiglu_fwd")
@@ -567,6 +595,21 @@ def _rope_backward(ctx, dy):
 torch.library.register_autograd("maltos::rope", _rope_backward, setup_context=_rope_setup)
 
 
+def _rope_pair_setup(ctx, inputs, output):
+    _xa, _xb, cos, sin, positions, position_offset, inverse = inputs
+    ctx.save_for_backward(cos, sin, positions)
+    ctx.position_offset, ctx.inverse = position_offset, inverse
+
+
+def _rope_pair_backward(ctx, dya, dyb):
+    cos, sin, positions = ctx.saved_tensors
+    dxa, dxb = torch.ops.maltos.rope_pair(dya, dyb, cos, sin, positions, ctx.position_offset, not ctx.inverse)
+    return dxa, dxb, None, None, None, None, None
+
+
+torch.library.register_autograd("maltos::rope_pair", _rope_pair_backward, setup_context=_rope_pair_setup)
+
+
 def _swiglu_setup(ctx, inputs, output):
     ctx.save_for_backward(*inputs)
 
@@ -627,6 +670,12 @@ def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, 
 def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, positions: torch.Tensor | None = None,
          position_offset: int = 0) -> torch.Tensor:
     return torch.ops.maltos.rope(x, cos, sin, positions, int(position_offset), False)
+
+
+def rope_pair(xa: torch.Tensor, xb: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, positions: torch.Tensor | None = None,
+              position_offset: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
+    """rope(xa), rope(xb) from one kernel launch (and one in the backward): bit-equal to two `rope` calls."""
+    return torch.ops.maltos.rope_pair(xa, xb, cos, sin, positions, int(position_offset), False)
 
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -118,6 +118,41 @@ def test_rope_forward_backward(dev, dtype, use_ids):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_ids", [False, True])
+def test_rope_pair_equals_two_rotations(dev, dtype, use_ids):
+    """q and k of a GQA layer (models/llama.py:143-144) rotated by one launch: the oracle's values for each operand, bit
+    for bit what two single launches give, forward and backward, on the strided views the model hands over."""
+    B, Hq, Hk, S, D = 2, 6, 2, 19, 64
+    g = torch.Generator().manual_seed(7)
+    mk = lambda h: torch.randn(B, S, h, D, generator=g).to(dtype).transpose(1, 2)
+    xq, xk, dq, dk = mk(Hq), mk(Hk), mk(Hq), mk(Hk)
+    cos_t, sin_t = ol.rope_tables(D, 64)
+    cos_t, sin_t = cos_t.to(dtype), sin_t.to(dtype)
+    pos = torch.stack([torch.arange(S) % 5, torch.arange(S) + 3]) if use_ids else None
+    cos, sin = ol.rope_cos_sin(cos_t, sin_t, seq_len=S, position_offset=2, position_ids=pos)
+    kw = dict(positions=None if pos is None else pos.to(dev), position_offset=2)
+    qg, kg = xq.to(dev).requires_grad_(True), xk.to(dev).requires_grad_(True)
+    yq, yk = ops.rope_pair(qg, kg, cos_t.to(dev), sin_t.to(dev), **kw)
+    assert yq.stride() == qg.stride() and yk.stride() == kg.stride()
+    (yq * dq.to(dev)).sum().backward(retain_graph=True)
+    (yk * dk.to(dev)).sum().backward()
+    q1, k1 = xq.to(dev).requires_grad_(True), xk.to(dev).requires_grad_(True)
+    sq, sk = ops.rope(q1, cos_t.to(dev), sin_t.to(dev), **kw), ops.rope(k1, cos_t.to(dev), sin_t.to(dev), **kw)
+    sq.backward(dq.to(dev))
+    sk.backward(dk.to(dev))
+    for got, single in ((yq, sq), (yk, sk), (qg.grad, q1.grad), (kg.grad, k1.grad)):
+        assert torch.equal(got, single)
+    for got, x, d in ((yq, xq, None), (yk, xk, None), (qg.grad, None, dq), (kg.grad, None, dk)):
+        want = ol.apply_rotary(x, cos, sin) if d is None else ol.apply_rotary_backward(d, cos, sin)
+        if dtype == torch.float32:
+            torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-6)
+        else:
+            assert torch.equal(got.cpu(), want)
+    with pytest.raises(ValueError):
+        ops.rope_pair(qg, kg[:, :, :5], cos_t.to(dev), sin_t.to(dev))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n", [(5, 7), (64, 1376)])
 def test_swiglu_forward_backward(dev, dtype, n):
     g = torch.Generator().manual_seed(sum(n))
