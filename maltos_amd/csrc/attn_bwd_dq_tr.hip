@@ -80,6 +80,10 @@ __device__ __forceinline__ void wait_lgkm(v2i32 (&x)[8]) {
                : "n"(N));
 }
 template <int N>
+__device__ __forceinline__ void wait_lgkm(v4i32 (&x)[1]) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(x[0]) : "n"(N));
+}
+template <int N>
 __device__ __forceinline__ void wait_lgkm(v4i32 (&x)[2]) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(x[0]), "+v"(x[1]) : "n"(N));
 }
@@ -256,19 +260,38 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   // ---- per-lane LDS read offsets (tile invariant) ----
   // (LDS addresses of stage 0; the stage, the key block and the tile are added as instruction offsets)
-  uint32_t ra[KS];  // row-major fragment (A operand): row l32 (+32 kb), chunk 2 ks + hh
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) ra[ks] = lds0 + l32 * RB + (((ks * 2 + hh) ^ swz<D>(l32 & 15)) << 4);
-  uint32_t ta[2][DB];  // K^T fragment halves: key row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4)
+  // Row-major fragment (A operand): row l32 (+32 kb), chunk 2 ks + hh.  K^T fragment halves: key row 16 c + 8 part + 4 hh
+  // + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4).  The chunk swizzle is an XOR, so chunk (2 ks + hh) ^ s is
+  // ((ks ^ s/2) * 2) | ((hh ^ s) & 1) and column chunk (4 db + y) ^ s is ((db ^ s/4) * 4) | (y ^ s % 4): an address is a
+  // per-lane base plus an XOR of a compile-time index with a per-lane constant.  Without a document mask the sixteen
+  // addresses are kept in registers; with one the kernel needs those registers (it otherwise spills into the tile
+  // loop) and forms each address where it is used, two instructions each.
+  constexpr bool ADDR_IN_REGS = MODE != MLTS_MASK_DOC;
+  const uint32_t ra_base = lds0 + l32 * RB + (((hh ^ swz<D>(l32 & 15)) & 1) << 4);
+  const uint32_t ra_x = static_cast<uint32_t>(swz<D>(l32 & 15) >> 1);
+  uint32_t ta_base[2], ta_x[2];
 #pragma unroll
   for (int part = 0; part < 2; ++part) {
     const int rlow = part * 8 + hh * 4 + (l16 >> 2);
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
-      ta[part][db] = lds0 + rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
-    }
+    const int col0 = (l32 >> 4) * 16 + (l16 & 3) * 4;  // column inside a 32-column block
+    ta_base[part] = lds0 + rlow * RB + ((((col0 >> 3) ^ swz<D>(rlow)) & 3) << 4) + ((col0 >> 2) & 1) * 8;
+    ta_x[part] = static_cast<uint32_t>(swz<D>(rlow) >> 2);
   }
+  uint32_t ra_reg[KS], ta_reg[2][DB];
+  if (ADDR_IN_REGS) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ra_reg[ks] = ra_base + ((static_cast<uint32_t>(ks) ^ ra_x) << 5);
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) ta_reg[part][db] = ta_base[part] + ((static_cast<uint32_t>(db) ^ ta_x[part]) << 6);
+  }
+  auto ra = [&](const int ks) -> uint32_t {
+    return ADDR_IN_REGS ? ra_reg[ks] : ra_base + ((static_cast<uint32_t>(ks) ^ ra_x) << 5);
+  };
+  auto ta = [&](const int part, const int db) -> uint32_t {
+    return ADDR_IN_REGS ? ta_reg[part][db] : ta_base[part] + ((static_cast<uint32_t>(db) ^ ta_x[part]) << 6);
+  };
 
   bf16x8 qf[KS], ndof[KS];  // Q and -dO fragments (B operands): row 32 wave + l32, the row-major fragment pattern
   {
@@ -287,8 +310,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     v4i32 fq[KS], fd[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      fq[ks] = lds_read_b128<0>(ra[ks] + wave * (32 * RB));
-      fd[ks] = lds_read_b128<0>(ra[ks] + wave * (32 * RB) + BM * RB);
+      fq[ks] = lds_read_b128<0>(ra(ks) + wave * (32 * RB));
+      fd[ks] = lds_read_b128<0>(ra(ks) + wave * (32 * RB) + BM * RB);
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -321,16 +344,16 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   // read groups are kept small (two 16-byte row reads, or four transpose reads) and two are in flight: the kernel
   // sits at the 256-register limit of two wavefronts per SIMD
 #define MLTS_RREAD2(dst, KB, KS0)                                                  \
-  dst[0] = lds_read_b128<(KB) * 32 * RB>(ra[(KS0)] + so);                             \
-  dst[1] = lds_read_b128<TILE_BYTES + (KB) * 32 * RB>(ra[(KS0)] + so);
+  dst[0] = lds_read_b128<(KB) * 32 * RB>(ra((KS0)) + so);                             \
+  dst[1] = lds_read_b128<TILE_BYTES + (KB) * 32 * RB>(ra((KS0)) + so);
 #define MLTS_SMFMA2(src, KS0)                                                                            \
   s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), qf[(KS0)], s, 0, 0, 0);                   \
   dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), ndof[(KS0)], dp, 0, 0, 0);
 #define MLTS_TREAD4(dst, C, H)                                                       \
-  dst[0] = lds_read_tr16_b64<(C) * 16 * RB>(ta[0][2 * (H)] + so);                       \
-  dst[1] = lds_read_tr16_b64<(C) * 16 * RB>(ta[1][2 * (H)] + so);                       \
-  dst[2] = lds_read_tr16_b64<(C) * 16 * RB>(ta[0][2 * (H) + 1] + so);                   \
-  dst[3] = lds_read_tr16_b64<(C) * 16 * RB>(ta[1][2 * (H) + 1] + so);
+  dst[0] = lds_read_tr16_b64<(C) * 16 * RB>(ta(0, 2 * (H)) + so);                       \
+  dst[1] = lds_read_tr16_b64<(C) * 16 * RB>(ta(1, 2 * (H)) + so);                       \
+  dst[2] = lds_read_tr16_b64<(C) * 16 * RB>(ta(0, 2 * (H) + 1) + so);                   \
+  dst[3] = lds_read_tr16_b64<(C) * 16 * RB>(ta(1, 2 * (H) + 1) + so);
 #define MLTS_TMFMA2(src, H, BFRAG)                                                                                        \
   dqacc[2 * (H)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0], src[1]), BFRAG, dqacc[2 * (H)], 0, 0, 0);       \
   dqacc[2 * (H) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2], src[3]), BFRAG, dqacc[2 * (H) + 1], 0, 0, 0);
@@ -348,18 +371,25 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       const uint32_t ma = lds0 + C::META_OFF + (so / STAGE_BYTES) * C::META_BYTES + (kb * 32 + hh * 4) * 4;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        v4i32 kp[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [0] positions, [1] sequence ids of keys kb * 32 + g * 8 + hh * 4 .. + 3
         if (MODE == MLTS_MASK_DOC) {
+          // positions first, then sequence ids through the same registers
+          v4i32 kp[1];
           kp[0] = g == 0 ? lds_read_b128<0>(ma) : g == 1 ? lds_read_b128<32>(ma) : g == 2 ? lds_read_b128<64>(ma) : lds_read_b128<96>(ma);
-          kp[1] = g == 0 ? lds_read_b128<BN * 4>(ma) : g == 1 ? lds_read_b128<BN * 4 + 32>(ma) : g == 2 ? lds_read_b128<BN * 4 + 64>(ma) : lds_read_b128<BN * 4 + 96>(ma);
           wait_lgkm<0>(kp);
-        }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
-          bool vis = kb * 32 + g * 8 + r <= klim_t;
-          if (MODE == MLTS_MASK_DOC) vis = vis && (kp[0][r] <= qpos) && (kp[1][r] == qseq) && (qseq >= 0);
-          if (!vis) s[g * 4 + r] = -INFINITY;
+          for (int r = 0; r < 4; ++r)
+            if (!(kb * 32 + g * 8 + r <= klim_t && kp[0][r] <= qpos && qseq >= 0)) s[g * 4 + r] = -INFINITY;
+          kp[0] = g == 0 ? lds_read_b128<BN * 4>(ma) : g == 1 ? lds_read_b128<BN * 4 + 32>(ma) : g == 2 ? lds_read_b128<BN * 4 + 64>(ma) : lds_read_b128<BN * 4 + 96>(ma);
+          wait_lgkm<0>(kp);
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (kp[0][r] != qseq) s[g * 4 + r] = -INFINITY;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
+            if (!(kb * 32 + g * 8 + r <= klim_t)) s[g * 4 + r] = -INFINITY;
+          }
         }
       }
     };

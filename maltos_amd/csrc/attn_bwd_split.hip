@@ -297,21 +297,36 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 
   // ---- per-lane LDS offsets (tile invariant) ----
   const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem)));
-  int roff[KS];  // row-major fragment (A operand): row l32 (+32 qb), chunk 2 ks + hh; role 0 reads Q, role 1 dO
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    roff[ks] = role * TILE_BYTES + l32 * RB + (((ks * 2 + hh) ^ swz<D>(l32 & 15)) << 4);
-  int toff[2][DB];  // transposed fragment halves: query row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16)
-                    // + 4 (l16%4); role 0 reads dO^T, role 1 Q^T
+  // Row-major fragment (A operand): row l32 (+32 qb), chunk 2 ks + hh; role 0 reads Q, role 1 dO.  Transposed fragment
+  // halves: query row 16 c + 8 part + 4 hh + l16/4, columns 32 db + 16 (l32/16) + 4 (l16%4); role 0 reads dO^T, role 1
+  // Q^T.  The chunk swizzle is an XOR, so chunk (2 ks + hh) ^ s is ((ks ^ s/2) * 2) | ((hh ^ s) & 1) and column chunk
+  // (4 db + y) ^ s is ((db ^ s/4) * 4) | (y ^ s % 4): an offset is a per-lane base plus an XOR of a compile-time index
+  // with a per-lane constant.  With a document mask the kernel needs the registers of the sixteen offsets (it
+  // otherwise spills into the tile loop) and forms them per tile from the six values they derive from.
+  constexpr bool OFFS_IN_REGS = MODE == MLTS_MASK_CAUSAL;
+  const int roff_base = role * TILE_BYTES + l32 * RB + (((hh ^ swz<D>(l32 & 15)) & 1) << 4);
+  const int roff_x = swz<D>(l32 & 15) >> 1;
+  int toff_base[2], toff_x[2];
 #pragma unroll
   for (int part = 0; part < 2; ++part) {
     const int rlow = part * 8 + hh * 4 + (l16 >> 2);
-#pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      const int col = db * 32 + (l32 >> 4) * 16 + (l16 & 3) * 4;
-      toff[part][db] = (1 - role) * TILE_BYTES + rlow * RB + (((col >> 3) ^ swz<D>(rlow)) << 4) + ((col >> 2) & 1) * 8;
-    }
+    const int col0 = (l32 >> 4) * 16 + (l16 & 3) * 4;  // column inside a 32-column block
+    toff_base[part] = (1 - role) * TILE_BYTES + rlow * RB + ((((col0 >> 3) ^ swz<D>(rlow)) & 3) << 4) + ((col0 >> 2) & 1) * 8;
+    toff_x[part] = swz<D>(rlow) >> 2;
   }
+  int roff_reg[KS], toff_reg[2][DB];
+  if (OFFS_IN_REGS) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) roff_reg[ks] = roff_base + ((ks ^ roff_x) << 5);
+#pragma unroll
+    for (int part = 0; part < 2; ++part)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) toff_reg[part][db] = toff_base[part] + ((db ^ toff_x[part]) << 6);
+  }
+  auto roff = [&](const int ks) -> int { return OFFS_IN_REGS ? roff_reg[ks] : roff_base + ((ks ^ roff_x) << 5); };
+  auto toff = [&](const int part, const int db) -> int {
+    return OFFS_IN_REGS ? toff_reg[part][db] : toff_base[part] + ((db ^ toff_x[part]) << 6);
+  };
   // statistics of rows 32 qb + 8 g + 4 hh .. +3: role 0 reads lse2, role 1 delta
   const int soff_lane = STAT_OFF + role * (BQ * 4) + hh * 16;
   const uint32_t pbuf_lane = lds0 + PBUF_OFF + kb * PBUF_BYTES + lane * 16;
@@ -350,13 +365,13 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
     uint32_t ra[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
+    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff(ks);
     const uint32_t sa = sb + soff_lane;
     uint32_t ta[2][DB];
 #pragma unroll
     for (int part = 0; part < 2; ++part)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff(part, db);
     const int causal_t = kj - p.causal_off - q0 - hh * 4;
 
     bf16x8 pfr[2][2];
@@ -527,7 +542,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
     uint32_t ra[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff[ks];
+    for (int ks = 0; ks < KS; ++ks) ra[ks] = sb + roff(ks);
     const uint32_t sa = sb + soff_lane;
     v4i32 st[8], g0[4], g1[4];
 #pragma unroll
@@ -614,7 +629,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 #pragma unroll
     for (int part = 0; part < 2; ++part)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff[part][db];
+      for (int db = 0; db < DB; ++db) ta[part][db] = sb + toff(part, db);
     v2i32 h0[8], h1[8];
     if constexpr (D == 128) {
       MLTS_TREAD8(h0, 0)
