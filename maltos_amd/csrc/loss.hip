@@ -50,8 +50,8 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restric
 // STAGED: the row lives in dynamic LDS between the passes; otherwise it is re-read from global
 // memory (L2) -- used only when a row does not fit.
 template <typename T, bool STAGED, bool VEC>
-__global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* __restrict__ logits,
-                                                            const int64_t* __restrict__ labels, T* __restrict__ dlogits,
+__global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* logits,  // may be dlogits (gradient in place)
+                                                            const int64_t* __restrict__ labels, T* dlogits,
                                                             float* __restrict__ row_loss,
                                                             const int32_t* __restrict__ count, int vocab,
                                                             int64_t ignore_index) {
@@ -111,10 +111,13 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* __restrict_
   } else {
     for (int c = threadIdx.x; c < vocab; c += kCeThreads) se += exp2f(to_f32<T>(src[c]) * kLog2e - mxs);
   }
+  // read before the barrier inside block_sum: behind it other threads may already be storing gradients over the row
+  float label_logit = 0.f;
+  if (threadIdx.x == 0 && label_ok) label_logit = to_f32<T>(src[label]);
   se = block_sum(se, red);
   const float lse = mx + logf(se);
   if (threadIdx.x == 0) {
-    row_loss[row] = label_ok ? lse - to_f32<T>(src[label]) : NAN;
+    row_loss[row] = label_ok ? lse - label_logit : NAN;
   }
 
   // pass 3: gradient
@@ -149,8 +152,8 @@ __global__ __launch_bounds__(kCeThreads) void ce_row_kernel(const T* __restrict_
 // flight per CU instead of the two that fit when rows are staged in LDS (six wavefronts per SIMD = three blocks per CU
 // is the register budget that still compiles without spills for eight vectors per lane).
 template <typename T, int NV>
-__global__ __launch_bounds__(kCeThreads, 6) void ce_row_reg_kernel(const T* __restrict__ logits,
-                                                                const int64_t* __restrict__ labels, T* __restrict__ dlogits,
+__global__ __launch_bounds__(kCeThreads, 6) void ce_row_reg_kernel(const T* logits,  // may be dlogits (gradient in place)
+                                                                const int64_t* __restrict__ labels, T* dlogits,
                                                                 float* __restrict__ row_loss,
                                                                 const int32_t* __restrict__ count, int vocab,
                                                                 int64_t ignore_index) {

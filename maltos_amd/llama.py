@@ -291,7 +291,8 @@ class LlamaForCausalLM(nn.Module):
             return logits
         if input_ids is not None and labels.shape != input_ids.shape:
             raise ValueError(f"labels shape must match input_ids shape, got {labels.shape} vs {input_ids.shape}")
-        loss = causal_cross_entropy(logits, labels)
+        # the logits are this function's own and are not returned with the loss: their gradient may take their place
+        loss = causal_cross_entropy(logits, labels, overwrite_logits=logits.is_cuda and logits.is_contiguous())
         return loss if loss_weight is None else loss * float(loss_weight)
 
     def context_parallel_spec(self) -> list[str]:

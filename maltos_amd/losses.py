@@ -14,5 +14,7 @@ from . import ops
 from .constants import IGNORE_INDEX
 
 
-def causal_cross_entropy(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
-    return ops.cross_entropy(logits, labels, IGNORE_INDEX)
+def causal_cross_entropy(logits: torch.Tensor, labels: torch.Tensor, *, overwrite_logits: bool = False) -> torch.Tensor:
+    """overwrite_logits: the caller owns the logits and never reads them again; their gradient then replaces them in
+    the same buffer (no second logits-sized tensor, and the kernel streams faster over one buffer than over two)."""
+    return ops.cross_entropy(logits, labels, IGNORE_INDEX, overwrite_logits=overwrite_logits)

@@ -365,14 +365,17 @@ def _swiglu_bwd(dh, gate, up):
     return dg, du
 
 
-def _ce_fwd_bwd(logits, labels, ignore_index):
+def _ce_fwd_bwd(logits, labels, ignore_index, overwrite: bool = False):
+    """overwrite: the gradient replaces the logits in their own buffer (they must be contiguous)."""
     _require_gpu(logits, labels)
     vocab = logits.size(-1)
     lg = logits.contiguous().view(-1, vocab)
     lb = labels.contiguous().view(-1).to(torch.int64)
     if lb.numel() != lg.size(0):
         raise ValueError(f"labels ({lb.numel()}) do not match logits rows ({lg.size(0)})")
-    dlogits = torch.empty_like(lg)
+    if overwrite and lg.data_ptr() != logits.data_ptr():
+        raise ValueError("cross_entropy(overwrite_logits=True) needs contiguous logits")
+    dlogits = lg if overwrite else torch.empty_like(lg)
     loss = torch.empty((), dtype=torch.float32, device=logits.device)
     count = torch.empty((), dtype=torch.int32, device=logits.device)
     L = _lib.lib()
@@ -659,6 +662,30 @@ def _ce_backward(ctx, dloss, _ddlogits, _dcount):
 torch.library.register_autograd("maltos::ce_fwd_bwd", _ce_backward, setup_context=_ce_setup)
 
 
+class _CrossEntropyOverLogits(torch.autograd.Function):
+    """The loss whose gradient replaces the logits in their buffer: one read and one write of the same addresses (the
+    kernel then streams at the rate of an in-place update instead of a copy's) and no second logits-sized tensor.  For
+    callers that own the logits and never look at them again; a plain autograd function because an operator that
+    overwrites an argument it is differentiated by has no functional form to register."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, ignore_index):
+        loss, dlogits, _count = _ce_fwd_bwd(logits.detach(), labels, ignore_index, overwrite=True)
+        ctx.save_for_backward(dlogits)
+        ctx.consumed = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, dloss):
+        if ctx.consumed:
+            raise RuntimeError("cross_entropy(overwrite_logits=True): backward ran twice through the same loss; its logits "
+                               "gradient is scaled in place by the first pass, so recompute the loss instead")
+        (dlogits,) = ctx.saved_tensors
+        torch.ops.maltos.scale_by_scalar_(dlogits, dloss)
+        ctx.consumed = True
+        return dlogits, None, None
+
+
 # --------------------------------------------------------------------------------------------
 # public differentiable entry points
 # --------------------------------------------------------------------------------------------
@@ -696,8 +723,12 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.ops.maltos.swiglu_fwd(gate, up)
 
 
-def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100) -> torch.Tensor:
-    """fp32 scalar: sum CE over supervised rows / max(1, #supervised rows)."""
+def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100, *,
+                  overwrite_logits: bool = False) -> torch.Tensor:
+    """fp32 scalar: sum CE over supervised rows / max(1, #supervised rows).  overwrite_logits=True lets the gradient take
+    the place of the (contiguous) logits, which the caller must not read afterwards."""
+    if overwrite_logits:
+        return _CrossEntropyOverLogits.apply(logits, labels, int(ignore_index))
     return torch.ops.maltos.ce_fwd_bwd(logits, labels, int(ignore_index))[0]
 
 

@@ -216,6 +216,36 @@ def test_cross_entropy_backward_consumes_its_buffer_once(dev):
         loss.backward()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,vocab", [(7, 1000), (48, 32000), (3, 70001)])
+def test_cross_entropy_over_its_logits(dev, dtype, rows, vocab):
+    """overwrite_logits=True: the same loss and the same gradient, bit for bit, as the form with its own gradient
+    buffer, and the gradient stands where the logits stood (every row-kernel form: registers, LDS, re-read)."""
+    g = torch.Generator().manual_seed(rows + vocab)
+    logits = (3 * torch.randn(rows, vocab, generator=g)).to(dtype)
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    labels[1::4] = -100
+    a = logits.to(dev).requires_grad_(True)
+    (ops.cross_entropy(a, labels.to(dev)) * 0.5).backward()
+    base = logits.to(dev)
+    b = base.clone().requires_grad_(True)
+    owned = b * 1                      # a non-leaf the loss may consume, as the model's logits are
+    store = owned.data_ptr()
+    loss_b = ops.cross_entropy(owned, labels.to(dev), overwrite_logits=True)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    (loss_b * 0.5).backward(retain_graph=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() - before <= b.numel() * b.element_size() + 4096   # b.grad only
+    assert loss_b.item() == ops.cross_entropy(logits.to(dev), labels.to(dev)).item()
+    assert torch.equal(b.grad, a.grad)
+    assert owned.data_ptr() == store and torch.equal(owned.detach(), a.grad)
+    with pytest.raises(RuntimeError, match="backward ran twice"):
+        loss_b.backward()
+    with pytest.raises(ValueError, match="contiguous"):
+        ops.cross_entropy(base.t().contiguous().t(), labels.to(dev), overwrite_logits=True)
+
+
 def test_cross_entropy_without_targets_is_zero(dev):
     lg = torch.randn(2, 3, 5, device=dev, requires_grad=True)
     loss = ops.cross_entropy(lg, torch.full((2, 3), -100, device=dev))
