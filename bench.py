@@ -291,6 +291,8 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
     ang = torch.arange(2048, dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(0, 64, 2, dtype=torch.float32) / 64))[None, :]
     cos, sin = torch.cos(ang).to(bf).to(dev), torch.sin(ang).to(bf).to(dev)
     logits = rnd(N, V)
+    logits_own = rnd(N, V)                                          # overwritten by its own gradient, call after call
+    q2 = rnd(8, 2048, 8, 64).transpose(1, 2)
     labels = torch.randint(0, V, (N,), generator=g).to(dev)
     n_par = 58_073_600
     gsrc = torch.randn(n_par, device=dev).to(bf)
@@ -311,6 +313,9 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
         ("swiglu_fwd", "swiglu_fwd", 3 * N * I * e, lambda: torch.ops.maltos.swiglu_fwd(gate, up)),
         ("swiglu_bwd", "swiglu_bwd", 5 * N * I * e, lambda: torch.ops.maltos.swiglu_bwd(dh, gate, up)),
         ("cross_entropy_fwd_bwd", "ce", 2 * N * V * e, lambda: torch.ops.maltos.ce_fwd_bwd(logits, labels, -100)),
+        # the form the model uses for the logits it owns: the gradient takes their place (one buffer instead of two)
+        ("cross_entropy_fwd_bwd_over_logits", "ce", 2 * N * V * e, lambda: ops._ce_fwd_bwd(logits_own, labels, -100, overwrite=True)),
+        ("rope_pair_q_and_k", "rope", 2 * 2 * e * q.numel(), lambda: ops.rope_pair(q, q2, cos, sin)),
         ("grad_to_f32_with_norm", "grad_to_f32", 6 * n_par, lambda: ops.grad_to_f32_(gdst, gsrc, sq_out=sq)),
         ("attn_merge", "attn_merge", 10 * B4 * H4 * S4 * D4 + 12 * B4 * H4 * S4,
          lambda: ops.attention_merge_(out_acc, lse_acc, o_blk, lse_blk)),
