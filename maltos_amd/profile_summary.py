@@ -99,7 +99,8 @@ def hbm_traffic(raw: str, out_dir: str) -> bool:
     stat = B * H * S * 4 / 1e6             # one fp32 row statistic, MB
     ds = B * H * S * S / 2 * 2 / 1e6       # handed-over dS: 2 bytes per visible (query, key) pair
     alg = {"attn_fwd_dma_kernel": (3 * t, t + stat), "attn_bwd_dkdv_split_kernel": (4 * t + 2 * stat, 2 * t),
-           "attn_bwd_dq_tr_kernel": (4 * t + 2 * stat, t), "attn_bwd_dq_ds_kernel": (t + ds, t), "attn_delta_vec_kernel": (2 * t, stat)}
+           # the recomputing dQ kernel also reads O and writes the two row statistics (delta, LSE in base 2)
+           "attn_bwd_dq_tr_kernel": (5 * t + stat, t + 2 * stat), "attn_bwd_dq_ds_kernel": (t + ds, t), "attn_delta_vec_kernel": (2 * t, stat)}
     rec = {}
     with open(os.path.join(out_dir, "attn_cfg2_hbm_traffic.md"), "w") as f:
         f.write("# HBM traffic of the attention kernels, causal B=4 H=16 S=4096 D=128 bf16 (rocprofv3 --pmc)\n\n")
@@ -197,8 +198,9 @@ def main() -> int:
                     "rocprofv3 kernel statistics of the headline step (causal attention fwd+bwd, B=4 H=16 S=4096 D=128 bf16)",
                     "rocprofv3 --kernel-trace --stats -f csv -d <raw dir>/stats -- python3 bench.py --steps 40 --warmup 10 --skip-cpu --skip-extra",
                     "Source: `*_kernel_stats.csv` of that run.  `attn_fwd_dma_kernel` = `attn_fwd`, `attn_bwd_dkdv_split_kernel` = `attn_bwd_dkdv`,\n"
-                    "`attn_bwd_dq_tr_kernel` = `attn_bwd_dq` (the recomputing dQ kernel of the default backward), `attn_delta_vec_kernel` = `attn_delta`\n"
-                    "in bench.py's `kernels` block, whose HIP-event averages these agree with.", top=8):
+                    "`attn_bwd_dq_tr_kernel` = `attn_bwd_dq` (the recomputing dQ kernel of the default backward; it runs first and also\n"
+                    "forms the row statistics delta and LSE in base 2, so no separate delta pass appears) in bench.py's `kernels` block,\n"
+                    "whose HIP-event averages these agree with.", top=8):
         done.append("attn_cfg2_kernel_stats.md")
     if kernel_stats(args.raw, "llama", os.path.join(args.out, "llama50m_step_kernel_stats.md"),
                     "rocprofv3 kernel statistics of the LLaMA-50M bf16 train step (B=8, S=2048; configuration 5)",
