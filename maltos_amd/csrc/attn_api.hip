@@ -49,19 +49,10 @@ const char* shape_problem(const mlts_attn_shape* s) {
   return nullptr;
 }
 
-// queries and keys of a document-mask call are the same tokens (self-attention over packed rows)
-bool same_tokens(const mlts_attn_shape* s) {
-  return s->Sq == s->Sk && s->q_pos == s->k_pos && s->q_seq == s->k_seq;
-}
-
-int64_t run_bounds_bytes(const mlts_attn_shape* s) {
-  return same_tokens(s) ? 2 * align256(static_cast<int64_t>(s->B) * s->Sq * 4) + align256(static_cast<int64_t>(s->B) * 4) : 0;
-}
-
 int64_t stats_bytes(const mlts_attn_shape* s) {
   if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return 0;
   const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
-  return align256(s->B * nq * 16) + align256(s->B * nk * 16) + run_bounds_bytes(s);
+  return align256(s->B * nq * 16) + align256(s->B * nk * 16);
 }
 
 void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o,
@@ -91,7 +82,6 @@ void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const v
   p.k_seq = s->k_seq;
   p.q_stats = nullptr;
   p.k_stats = nullptr;
-  p.run_lo = p.run_hi = p.row_ok = nullptr;
   p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
   p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
   p.nqt = 0;
@@ -108,17 +98,6 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, char* ws, hipStream_t
   mlts_launch_tile_stats(s->k_pos, s->k_seq, s->B, s->Sk, kst, st);
   p.q_stats = qst;
   p.k_stats = kst;
-  if (same_tokens(s)) {
-    const int64_t n = align256(static_cast<int64_t>(s->B) * s->Sq * 4);
-    int32_t* lo = reinterpret_cast<int32_t*>(ws);
-    int32_t* hi = reinterpret_cast<int32_t*>(ws + n);
-    int32_t* ok = reinterpret_cast<int32_t*>(ws + 2 * n);
-    ws += run_bounds_bytes(s);
-    mlts_launch_run_bounds(s->q_pos, s->q_seq, s->B, s->Sq, lo, hi, ok, st);
-    p.run_lo = lo;
-    p.run_hi = hi;
-    p.row_ok = ok;
-  }
   return ws;
 }
 
@@ -332,63 +311,6 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
   if (threadIdx.x == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
 }
 
-
-// ---- run bounds of a packed row ----------------------------------------------------------------
-// One block per row; thread t owns the tokens [t * L, (t + 1) * L).  A run starts at token 0 and wherever the sequence
-// id changes.  run_lo[i] = start of i's run, run_hi[i] = last token of i's run; padding gets (INT_MAX, -1).  row_ok says
-// whether the row has the plain packed layout (see AttnParams); the kernels only use the bounds of such rows.
-__global__ __launch_bounds__(256) void run_bounds_kernel(const int32_t* __restrict__ pos, const int32_t* __restrict__ seq, int S,
-                                                         int32_t* __restrict__ run_lo, int32_t* __restrict__ run_hi,
-                                                         int32_t* __restrict__ row_ok) {
-  __shared__ int last_brk[256], first_brk[256], bad[256];
-  const int b = blockIdx.x, t = threadIdx.x;
-  const int32_t* ps = pos + static_cast<int64_t>(b) * S;
-  const int32_t* ss = seq + static_cast<int64_t>(b) * S;
-  int32_t* lo = run_lo + static_cast<int64_t>(b) * S;
-  int32_t* hi = run_hi + static_cast<int64_t>(b) * S;
-  const int L = (S + 255) / 256;
-  const int i0 = min(t * L, S), i1 = min(i0 + L, S);
-  auto is_break = [&](int i) -> bool { return i == 0 || ss[i] != ss[i - 1]; };
-  int lb = -1, fb = 0x7fffffff, wrong = 0;
-  for (int i = i0; i < i1; ++i) {
-    if (is_break(i)) {
-      lb = i;
-      if (fb == 0x7fffffff) fb = i;
-    }
-    if (i > 0 && ss[i] >= 0) {
-      const bool same_run = ss[i] == ss[i - 1] && ps[i] == ps[i - 1] + 1;
-      const bool next_run = ss[i - 1] >= 0 && ss[i] > ss[i - 1];
-      if (!same_run && !next_run) wrong = 1;
-    }
-  }
-  last_brk[t] = lb;
-  first_brk[t] = fb;
-  bad[t] = wrong;
-  __syncthreads();
-  int carry_lo = -1, carry_hi = 0x7fffffff, any_bad = 0;
-  for (int u = 0; u < t; ++u) carry_lo = max(carry_lo, last_brk[u]);                 // last break before this segment
-  for (int u = 255; u > t; --u) carry_hi = min(carry_hi, first_brk[u]);              // first break after it
-  if (t == 0) {
-    for (int u = 0; u < 256; ++u) any_bad |= bad[u];
-    row_ok[b] = any_bad ? 0 : 1;
-  }
-  int cur = carry_lo;
-  for (int i = i0; i < i1; ++i) {
-    if (is_break(i)) cur = i;
-    lo[i] = ss[i] >= 0 ? cur : 0x7fffffff;
-  }
-  int nxt = carry_hi == 0x7fffffff ? S : carry_hi;  // index of the next run's first token
-  for (int i = i1 - 1; i >= i0; --i) {
-    hi[i] = ss[i] >= 0 ? nxt - 1 : -1;
-    if (is_break(i)) nxt = i;
-  }
-}
-
-void mlts_launch_run_bounds(const int32_t* pos, const int32_t* seq, int B, int S, int32_t* run_lo, int32_t* run_hi,
-                            int32_t* row_ok, hipStream_t st) {
-  if (B == 0 || S == 0) return;
-  hipLaunchKernelGGL(run_bounds_kernel, dim3(B), dim3(256), 0, st, pos, seq, S, run_lo, run_hi, row_ok);
-}
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
   const int ntiles = (S + kAttnTile - 1) / kAttnTile;

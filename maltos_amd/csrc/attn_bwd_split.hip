@@ -168,16 +168,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
   }
   const int4 wk_stats = MODE == MLTS_MASK_DOC ? ((kb >> 1) ? kstats[1] : kstats[0]) : make_int4(0, 0, 0, 0);
   int kpos = 0, kseq = -2;
-  // plain packed rows (see AttnParams::row_ok): key j is seen by exactly the queries j .. run_hi[j]
-  bool packed_row = false;
-  int k_run_hi = -1;
   if (MODE == MLTS_MASK_DOC && kj < p.Sk) {
     kpos = p.k_pos[static_cast<int64_t>(b) * p.Sk + kj];
     kseq = p.k_seq[static_cast<int64_t>(b) * p.Sk + kj];
-  }
-  if (MODE == MLTS_MASK_DOC && p.row_ok != nullptr) {
-    packed_row = __builtin_amdgcn_readfirstlane(p.row_ok[b]) != 0;
-    if (kj < p.Sk) k_run_hi = p.run_hi[static_cast<int64_t>(b) * p.Sk + kj];
   }
   // The walk over (query head of the group, query tile) is kept as two counters; a position past the end has
   // h == group.  (No division by the runtime tile count in the loop.)
@@ -389,18 +382,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       // hoisting all of them in front of the wave-uniform branch, where every tile would pay for them
       int causal_here = causal_t;
       asm volatile("" : "+v"(causal_here));
-      if (MODE == MLTS_MASK_DOC && packed_row) {
-        // plain packed row: the queries that see a key are an index range
-        const int lo_t = kj - q0 - hh * 4, hi_t = k_run_hi - q0 - hh * 4;
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int off = qb * 32 + g * 8 + r;
-            if (!(off >= lo_t && off <= hi_t)) s[g * 4 + r] = -INFINITY;
-          }
-        return;
-      }
       // document masks: positions and sequence ids of the queries come from the stage, four queries at a time
       const uint32_t ma = sb + STAT_OFF + 2 * BQ * 4 + (qb * 32 + hh * 4) * 4;
 #pragma unroll

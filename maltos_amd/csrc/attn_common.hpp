@@ -27,14 +27,6 @@ struct AttnParams {
   const int4* k_stats;  // [B, ceil(Sk/64)]
   int nq_stats, nk_stats;
   int nqt;              // query tiles per (batch, head) for the launched kernel
-  // MLTS_MASK_DOC with queries and keys described by the same id tensors (self-attention over one packed row), else
-  // null: run_lo / run_hi[B, S] = first / last index of the run of equal sequence ids a token belongs to (INT_MAX / -1
-  // for padding), row_ok[B] != 0 where the row has the plain packed layout (padding only at the end, sequence ids
-  // rising from run to run, positions rising by one inside a run).  In such a row query i sees key j iff
-  // run_lo[i] <= j <= i, i.e. j <= i <= run_hi[j]: a tile's mask needs no per-key or per-query ids.
-  const int32_t* run_lo;
-  const int32_t* run_hi;
-  const int32_t* row_ok;
 };
 
 // Backward-only extras.
@@ -138,5 +130,3 @@ __device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);
-void mlts_launch_run_bounds(const int32_t* pos, const int32_t* seq, int B, int S, int32_t* run_lo, int32_t* run_hi,
-                            int32_t* row_ok, hipStream_t st);

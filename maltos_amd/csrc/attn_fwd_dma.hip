@@ -127,17 +127,10 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   int qpos = 0, qseq = -1;
   int4 wq_stats = make_int4(0, -1, 0, -1);
   int4 bq_stats[BM / 64];
-  // plain packed rows (see AttnParams::row_ok): query i sees exactly the keys run_lo[i] .. i
-  bool packed_row = false;
-  int q_run_lo = 0x7fffffff;
   if (MODE == MLTS_MASK_DOC) {
     if (qrow < p.Sq) {
       qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qrow];
       qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qrow];
-    }
-    if (p.row_ok != nullptr) {
-      packed_row = __builtin_amdgcn_readfirstlane(p.row_ok[b]) != 0;
-      if (qrow < p.Sq) q_run_lo = p.run_lo[static_cast<int64_t>(b) * p.Sq + qrow];
     }
 #pragma unroll
     for (int w = 0; w < BM / 64; ++w) {
@@ -416,19 +409,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     __builtin_amdgcn_s_setprio(0);
     if (late && jn < j_end) sync();
     if (cls != TILE_SKIP) {
-      if (cls == TILE_MASKED && MODE == MLTS_MASK_DOC && packed_row) {
-        // plain packed row: the visible keys of a query are an index range
-        const int lo_t = q_run_lo - kv0 - hh * 4, hi_t = qrow - kv0 - hh * 4;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int off = kb * 32 + g * 8 + r;
-              if (!(off >= lo_t && off <= hi_t)) sacc[kb][g * 4 + r] = -INFINITY;
-            }
-      } else if (cls == TILE_MASKED) {
+      if (cls == TILE_MASKED) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
           // document masks: positions and sequence ids of this key block's 16 keys per lane half, read from the stage's

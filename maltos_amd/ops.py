@@ -81,20 +81,6 @@ def _ids32(t: torch.Tensor | None, batch: int, seq: int, what: str) -> torch.Ten
     return t.to(dtype=torch.int32).contiguous()
 
 
-def _same_ids(a: torch.Tensor | None, b: torch.Tensor | None) -> bool:
-    return (a is not None and b is not None and a.data_ptr() == b.data_ptr() and a.shape == b.shape
-            and a.stride() == b.stride() and a.dtype == b.dtype)
-
-
-def _ids32_pair(tq, tk, batch: int, sq: int, sk: int, what: str):
-    """int32 copies of the query-side and key-side ids; one tensor for both when they describe the same tokens
-    (self-attention), which is what lets the library see that through the pointers it is given."""
-    if sq == sk and _same_ids(tq, tk):
-        both = _ids32(tq, batch, sq, f"q_{what}")
-        return both, both
-    return _ids32(tq, batch, sq, f"q_{what}"), _ids32(tk, batch, sk, f"k_{what}")
-
-
 def _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq) -> AttnShape:
     s = AttnShape()
     s.B, s.Hq, s.Sq, s.D = q.size(0), q.size(1), q.size(2), q.size(3)
@@ -133,8 +119,8 @@ def attention_forward(q, k, v, *, mask_mode: int, scale: float | None = None, q_
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     if B == 0 or Sq == 0:
         return o, lse
-    q_pos, k_pos = _ids32_pair(q_pos, k_pos, B, Sq, k.size(2), "positions")
-    q_seq, k_seq = _ids32_pair(q_seq, k_seq, B, Sq, k.size(2), "sequence_ids")
+    q_pos, q_seq = _ids32(q_pos, B, Sq, "q_positions"), _ids32(q_seq, B, Sq, "q_sequence_ids")
+    k_pos, k_seq = _ids32(k_pos, B, k.size(2), "k_positions"), _ids32(k_seq, B, k.size(2), "k_sequence_ids")
     shape = _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
     L = _lib.lib()
     why = L.mlts_attn_supports(C.byref(shape))
@@ -178,8 +164,8 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
         raise ValueError(f"softmax_lse must be float32 of shape {(B, Hq, Sq)}, got {lse.dtype} {tuple(lse.shape)}")
     lse = lse.contiguous()
     scale = D ** -0.5 if scale is None else scale
-    q_pos, k_pos = _ids32_pair(q_pos, k_pos, B, Sq, Sk, "positions")
-    q_seq, k_seq = _ids32_pair(q_seq, k_seq, B, Sq, Sk, "sequence_ids")
+    q_pos, q_seq = _ids32(q_pos, B, Sq, "q_positions"), _ids32(q_seq, B, Sq, "q_sequence_ids")
+    k_pos, k_seq = _ids32(k_pos, B, Sk, "k_positions"), _ids32(k_seq, B, Sk, "k_sequence_ids")
     shape = _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
     L = _lib.lib()
     why = L.mlts_attn_supports(C.byref(shape))
