@@ -53,7 +53,9 @@ def bshd(B, H, S, D, gen, dtype):
     return torch.randn(B, S, H, D, generator=gen).to(dtype).transpose(1, 2)
 
 
-def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad_tail=0):
+def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad_tail=0, share_ids=True, ids=None):
+    """share_ids: queries and keys are described by the same id tensors (self-attention over packed rows) or by separate
+    copies (what a ring step or a gathered chunk passes).  ids = (positions, sequence_ids) overrides the drawn documents."""
     gen = torch.Generator().manual_seed(seed)
     q, k, v, do = bshd(B, Hq, Sq, D, gen, dtype), bshd(B, Hkv, Sk, D, gen, dtype), bshd(B, Hkv, Sk, D, gen, dtype), bshd(B, Hq, Sq, D, gen, dtype)
     kw, mask = {}, None
@@ -61,9 +63,10 @@ def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad
         mask = oa.causal_mask(Sq, Sk, "cpu")
     elif mode == ops.MASK_DOC:
         assert Sq == Sk
-        pos, seq = make_docs(B, Sq, gen, max_doc or max(2, Sq // 3), pad_tail)
+        pos, seq = ids if ids is not None else make_docs(B, Sq, gen, max_doc or max(2, Sq // 3), pad_tail)
         mask = oa.doc_mask(pos, pos, seq, seq)
-        kw = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+        dpos, dseq = pos.to(dev), seq.to(dev)
+        kw = dict(q_pos=dpos, k_pos=dpos if share_ids else pos.to(dev), q_seq=dseq, k_seq=dseq if share_ids else seq.to(dev))
     qf, kf, vf = (t.detach().float().clone().requires_grad_(True) for t in (q, k, v))
     want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
     want_o.backward(do.float())
@@ -120,6 +123,31 @@ def test_generic_head_dims(dev, D):
 def test_padding_rows_give_zeros_and_no_nan(dev, dtype):
     o, lse = run_case(dev, dtype, 2, 2, 2, 200, 200, 64, ops.MASK_DOC, seed=77, max_doc=50, pad_tail=37)
     assert not o[:, :, -37:].any() and (lse[:, :, -37:] == float("-inf")).all()
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_document_mask_irregular_rows(dev, D):
+    """The document mask is a rule on (query, key) pairs, whatever the row looks like: ids that fall, an id that returns
+    after another document, positions that restart or jump inside a run, padding in the middle, a zigzag order, next to
+    a regular packed row in the same batch; with shared and with separate id tensors.  All against the oracle's rule."""
+    S = 384
+    gen = torch.Generator().manual_seed(5 + D)
+    run_case(dev, torch.bfloat16, 2, 4, 2, S, S, D, ops.MASK_DOC, 21, max_doc=150, pad_tail=9, share_ids=False)
+    pos_r, seq_r = make_docs(1, S, gen, 120, pad_tail=5)
+    rows = [(pos_r[0], seq_r[0])]
+    idx = torch.arange(S)
+    rows.append((idx % 96, 3 - idx // 96))                                     # ids fall from run to run
+    rows.append((idx % 64, (idx // 64) % 2))                                   # ids 0,1,0,1,...: a document in several runs
+    rows.append((torch.where(idx < 200, idx, idx - 150), torch.zeros(S, dtype=torch.long)))  # positions restart inside a run
+    seq_pad = (idx // 100).clone()
+    seq_pad[150:170] = -1                                                      # padding in the middle
+    rows.append((idx % 100, seq_pad))
+    zig = torch.cat([idx[:96], idx[288:], idx[96:288]])                        # a chunk order that is not ascending
+    rows.append((zig, torch.zeros(S, dtype=torch.long)))
+    pos = torch.stack([r[0] for r in rows]).long()
+    seq = torch.stack([r[1] for r in rows]).long()
+    run_case(dev, torch.bfloat16, len(rows), 2, 1, S, S, D, ops.MASK_DOC, 22, ids=(pos, seq))
+    run_case(dev, torch.float32, len(rows), 2, 1, 96, 96, 32, ops.MASK_DOC, 23, ids=(pos[:, :96], seq[:, :96]))
 
 
 def test_reference_known_answers_through_hip(dev, known_answers):
