@@ -112,6 +112,19 @@ def test_forward_backward_parity(dev, dtype, case):
     run_case(dev, dtype, *case, seed=sum(case))
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_document_mask_many_tiles(dev, D):
+    """More than 64 and more than 128 key tiles per row: the kernels find the needed tiles 64 statistics entries at a
+    time, so the walk crosses chunk boundaries (and a ragged last tile) here; short documents make most tiles skippable,
+    one long document keeps whole chunks needed."""
+    run_case(dev, torch.bfloat16, 1, 2, 1, 4300, 4300, D, ops.MASK_DOC, 31 + D, max_doc=300, pad_tail=70)
+    S = 8400
+    idx = torch.arange(S)
+    seq = torch.where(idx < 5000, torch.zeros_like(idx), 1 + (idx - 5000) // 170)
+    pos = torch.where(idx < 5000, idx, (idx - 5000) % 170)
+    run_case(dev, torch.bfloat16, 1, 1, 1, S, S, D, ops.MASK_DOC, 32 + D, ids=(pos.view(1, S), seq.view(1, S)), share_ids=False)
+
+
 @pytest.mark.parametrize("D", [1, 3, 24, 96, 192])
 def test_generic_head_dims(dev, D):
     run_case(dev, torch.float32, 1, 2, 1, 70, 70, D, ops.MASK_CAUSAL, seed=D)
