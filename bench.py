@@ -57,10 +57,25 @@ def attention_inputs(torch, dev, B, H, S, D, seed=1234):
     return [torch.randn(B, H, S, D, generator=gen).bfloat16().to(dev) for _ in range(4)]
 
 
+PREHEAT_S = 0.25
+
+
+def preheat(torch, fn, seconds=PREHEAT_S):
+    """Untimed calls of the step for `seconds` of wall time, in front of the W warm-up steps: an idle GPU raises its
+    clocks over the first ~50 ms of load, which is longer than five warm-up steps of a 1.3 ms step (the first twenty
+    steps after five warm-up steps run 5 % slower than the twenty after them)."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+
+
 def timed(torch, fn, steps, warmup):
     """Mean seconds per call.  The interpreter's cyclic garbage collector is held off during the timed calls (as
     timeit does): one full collection is a 50-100 ms pause, which in a launch-bound loop of ten steps is the result."""
     import gc
+    preheat(torch, fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -87,6 +102,7 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(4, 16, 4096, 12
         o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_CAUSAL)
         state["grads"] = ops.attention_backward(do, q, k, v, o, lse, mask_mode=ops.MASK_CAUSAL)
 
+    preheat(torch, step)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -260,6 +276,7 @@ def bench_adamw(torch, ops, _lib, dev, steps, warmup):
         state["t"] += 1
         ops.adamw_step_(p, g, m, v, step=state["t"], p_lowp=lowp, **hp)
 
+    preheat(torch, step, 0.1)
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -324,6 +341,7 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
     out = {}
     with torch.no_grad():
         for label, timer, nbytes, fn in cases:
+            preheat(torch, fn, 0.05)
             for _ in range(3):
                 fn()
             torch.cuda.synchronize()
@@ -554,7 +572,8 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "causal self-attention fwd+bwd, B=4 H=16 S=4096 D=128, bf16 (configuration 2)",
-                   "flops_per_step": total_flops, "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS},
+                   "flops_per_step": total_flops, "frac_of_mfma_peak": value / MFMA_BF16_PEAK_TFLOPS,
+                   "preheat": f"{PREHEAT_S} s of untimed steps before the warm-up steps (clock ramp of an idle GPU)"},
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": dom["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": dom["tflops"] / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": measured_hbm_traffic().get(dominant),
