@@ -59,7 +59,27 @@ def test_rmsnorm_forward_backward(dev, dtype, rows, hidden):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,hidden", [(1, 256), (37, 512), (300, 1024), (4099, 2048)])
+@pytest.mark.parametrize("rows,hidden", [(4099, 512), (4101, 256), (5003, 1024)])
+def test_rmsnorm_many_narrow_rows(dev, dtype, rows, hidden):
+    """Millions of elements: every row is what the same row gives in a call of few rows (rows are independent), and the
+    oracle's values up to the rare second rounding flip that a different summation order of the mean allows."""
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = torch.randn(rows, hidden, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    xd, wd = x.to(dev), w.to(dev)
+    y = ops.rms_norm(xd, wd, 1e-5)
+    for lo, hi in ((0, 700), (rows - 301, rows), (2048, 2049)):
+        assert torch.equal(y[lo:hi], ops.rms_norm(xd[lo:hi].contiguous(), wd, 1e-5)), (lo, hi)
+    want = ol.rms_norm(x, w, 1e-5).float()
+    diff = (y.float().cpu() - want).abs()
+    tol = want.abs() * (1e-4 if dtype == torch.float32 else 2.0 ** -7) + 1e-6
+    assert (diff <= 2 * tol).all()
+    assert (diff > tol).float().mean().item() < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden", [(1, 256), (37, 512), (300, 1024), (4099, 2048), (4099, 512), (4102, 256),
+                                         (5001, 1024)])
 def test_add_rmsnorm_equals_add_then_rmsnorm(dev, dtype, rows, hidden):
     """The fused residual add + RMSNorm gives bit for bit what the two separate ops give, forward and backward, with
     the summed row used again downstream (the residual path) and without."""
