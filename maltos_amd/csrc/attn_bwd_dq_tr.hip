@@ -346,9 +346,17 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #define MLTS_RREAD2(dst, KB, KS0)                                                  \
   dst[0] = lds_read_b128<(KB) * 32 * RB>(ra((KS0)) + so);                             \
   dst[1] = lds_read_b128<TILE_BYTES + (KB) * 32 * RB>(ra((KS0)) + so);
+  // Two idle cycles behind every MFMA: a wavefront that streams MFMAs back to back keeps the SIMD's vector issue port,
+  // and the other wavefront of the SIMD (all eight do the same work, the older one of a pair wins every arbitration: it
+  // finishes a tile in 2800 cycles and waits 1500 at the barrier for the other's 4400) gets no vector instruction in.
+  // With the pause the other wavefront's exponentials go in between (measured: 3 % at head_dim 128, 4.5 % at 64; the
+  // same pause in the forward and dK/dV kernels, whose wavefronts run in different phases by construction, gave nothing).
+#define MLTS_MFMA_PAUSE(acc) asm volatile("s_nop 1" : "+v"(acc));
 #define MLTS_SMFMA2(src, KS0)                                                                            \
   s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0]), qf[(KS0)], s, 0, 0, 0);                   \
-  dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), ndof[(KS0)], dp, 0, 0, 0);
+  MLTS_MFMA_PAUSE(s)                                                                                     \
+  dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[1]), ndof[(KS0)], dp, 0, 0, 0);               \
+  MLTS_MFMA_PAUSE(dp)
 #define MLTS_TREAD4(dst, C, H)                                                       \
   dst[0] = lds_read_tr16_b64<(C) * 16 * RB>(ta(0, 2 * (H)) + so);                       \
   dst[1] = lds_read_tr16_b64<(C) * 16 * RB>(ta(1, 2 * (H)) + so);                       \
@@ -356,7 +364,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   dst[3] = lds_read_tr16_b64<(C) * 16 * RB>(ta(1, 2 * (H) + 1) + so);
 #define MLTS_TMFMA2(src, H, BFRAG)                                                                                        \
   dqacc[2 * (H)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[0], src[1]), BFRAG, dqacc[2 * (H)], 0, 0, 0);       \
-  dqacc[2 * (H) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2], src[3]), BFRAG, dqacc[2 * (H) + 1], 0, 0, 0);
+  MLTS_MFMA_PAUSE(dqacc[2 * (H)])                                                                                         \
+  dqacc[2 * (H) + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(src[2], src[3]), BFRAG, dqacc[2 * (H) + 1], 0, 0, 0); \
+  MLTS_MFMA_PAUSE(dqacc[2 * (H) + 1])
 
   // one 64-key tile for this wavefront's 32 queries, one 32-key block after the other; lane = query, accumulator
   // register e <-> key 32 kb + 8 (e/4) + 4 hh + e%4
@@ -460,6 +470,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #undef MLTS_SMFMA2
 #undef MLTS_TREAD4
 #undef MLTS_TMFMA2
+#undef MLTS_MFMA_PAUSE
 
   // ---- tile loop.  Barrier k: tile k is in LDS.  Tile k + 1 is fetched behind it into registers and stored into the
   // other stage (read last during tile k - 1) after the work on tile k.  There is one instance of the tile body
