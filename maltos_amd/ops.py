@@ -657,6 +657,9 @@ class _CrossEntropyOverLogits(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels, ignore_index):
         loss, dlogits, _count = _ce_fwd_bwd(logits.detach(), labels, ignore_index, overwrite=True)
+        # the kernel wrote through a raw pointer: tell autograd, so that another node that saved these logits for its
+        # own backward raises instead of differentiating through the gradient that now stands in their place
+        torch.autograd.graph.increment_version(logits)
         ctx.save_for_backward(dlogits)
         ctx.consumed = False
         return loss

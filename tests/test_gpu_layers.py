@@ -264,6 +264,13 @@ def test_cross_entropy_over_its_logits(dev, dtype, rows, vocab):
         loss_b.backward()
     with pytest.raises(ValueError, match="contiguous"):
         ops.cross_entropy(base.t().contiguous().t(), labels.to(dev), overwrite_logits=True)
+    # another consumer that saved the logits for its own backward is told that they are gone
+    c = base.clone().requires_grad_(True)
+    shared = c * 1
+    other = shared.sin().sum()
+    ops.cross_entropy(shared, labels.to(dev), overwrite_logits=True)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        other.backward()
 
 
 def test_cross_entropy_without_targets_is_zero(dev):
