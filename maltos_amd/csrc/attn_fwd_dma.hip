@@ -410,34 +410,56 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     if (late && jn < j_end) sync();
     if (cls != TILE_SKIP) {
       if (cls == TILE_MASKED) {
+        if constexpr (MODE == MLTS_MASK_DOC) {
+          // positions and sequence ids of the tile's keys (16 per key block and lane half; groups g = 0..3: keys
+          // kb * 32 + g * 8 + hh * 4 .. + 3) from the stage's copy, all sixteen reads at once: a read issued here waits
+          // out the LDS queue of the other wavefronts' fragment reads, and the second key block's ids travel while the
+          // first block's mask is applied
+          v4i32 kp[2][4], ksq[2][4];
+          const uint32_t ma = lds0 + META_OFF + stage * META_BYTES + (hh * 4) * 4;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          // document masks: positions and sequence ids of this key block's 16 keys per lane half, read from the stage's
-          // copy in one go (groups g = 0..3: keys kb * 32 + g * 8 + hh * 4 .. + 3)
-          v4i32 kp[4], ksq[4];
-          if (MODE == MLTS_MASK_DOC) {
-            const uint32_t ma = lds0 + META_OFF + stage * META_BYTES + (kb * 32 + hh * 4) * 4;
-            kp[0] = lds_read_b128<0>(ma);
-            kp[1] = lds_read_b128<32>(ma);
-            kp[2] = lds_read_b128<64>(ma);
-            kp[3] = lds_read_b128<96>(ma);
-            ksq[0] = lds_read_b128<BN * 4>(ma);
-            ksq[1] = lds_read_b128<BN * 4 + 32>(ma);
-            ksq[2] = lds_read_b128<BN * 4 + 64>(ma);
-            ksq[3] = lds_read_b128<BN * 4 + 96>(ma);
-            wait_lgkm<0>(kp[0], kp[1], kp[2], kp[3]);
-            wait_lgkm<0>(ksq[0], ksq[1], ksq[2], ksq[3]);
+          for (int kb = 0; kb < 2; ++kb) {
+            kp[kb][0] = kb ? lds_read_b128<128>(ma) : lds_read_b128<0>(ma);
+            kp[kb][1] = kb ? lds_read_b128<160>(ma) : lds_read_b128<32>(ma);
+            kp[kb][2] = kb ? lds_read_b128<192>(ma) : lds_read_b128<64>(ma);
+            kp[kb][3] = kb ? lds_read_b128<224>(ma) : lds_read_b128<96>(ma);
+            ksq[kb][0] = kb ? lds_read_b128<BN * 4 + 128>(ma) : lds_read_b128<BN * 4>(ma);
+            ksq[kb][1] = kb ? lds_read_b128<BN * 4 + 160>(ma) : lds_read_b128<BN * 4 + 32>(ma);
+            ksq[kb][2] = kb ? lds_read_b128<BN * 4 + 192>(ma) : lds_read_b128<BN * 4 + 64>(ma);
+            ksq[kb][3] = kb ? lds_read_b128<BN * 4 + 224>(ma) : lds_read_b128<BN * 4 + 96>(ma);
           }
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+          for (int kb = 0; kb < 2; ++kb) {
+            if (kb == 0) {
+              wait_lgkm<8>(kp[0][0], kp[0][1], kp[0][2], kp[0][3]);
+              wait_lgkm<8>(ksq[0][0], ksq[0][1], ksq[0][2], ksq[0][3]);
+            } else {
+              wait_lgkm<0>(kp[1][0], kp[1][1], kp[1][2], kp[1][3]);
+              wait_lgkm<0>(ksq[1][0], ksq[1][1], ksq[1][2], ksq[1][3]);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int kj = kbase + r;
-              bool vis = kj < p.Sk;
-              if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
-              if (MODE == MLTS_MASK_DOC) vis = vis && (kp[g][r] <= qpos) && (ksq[g][r] == qseq) && (qseq >= 0);
-              if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
+            for (int g = 0; g < 4; ++g) {
+              const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const bool vis = (kbase + r < p.Sk) && (kp[kb][g][r] <= qpos) && (ksq[kb][g][r] == qseq) && (qseq >= 0);
+                if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int kj = kbase + r;
+                bool vis = kj < p.Sk;
+                if (MODE == MLTS_MASK_CAUSAL) vis = vis && (kj <= qrow + p.causal_off);
+                if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
+              }
             }
           }
         }
