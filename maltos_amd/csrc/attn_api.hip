@@ -52,7 +52,9 @@ const char* shape_problem(const mlts_attn_shape* s) {
 int64_t stats_bytes(const mlts_attn_shape* s) {
   if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return 0;
   const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
-  return align256(s->B * nq * 16) + align256(s->B * nk * 16);
+  // tile statistics of both sides, then the visibility bits of the mixed (query group, key tile) pairs (512 bytes per
+  // pair, indexed densely: Sq * Sk / 8 bytes per batch row)
+  return align256(s->B * nq * 16) + align256(s->B * nk * 16) + align256(s->B * nq * nk * 512);
 }
 
 void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o,
@@ -82,6 +84,7 @@ void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const v
   p.k_seq = s->k_seq;
   p.q_stats = nullptr;
   p.k_stats = nullptr;
+  p.doc_bits = nullptr;
   p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
   p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
   p.nqt = 0;
@@ -98,6 +101,10 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, char* ws, hipStream_t
   mlts_launch_tile_stats(s->k_pos, s->k_seq, s->B, s->Sk, kst, st);
   p.q_stats = qst;
   p.k_stats = kst;
+  unsigned long long* bits = reinterpret_cast<unsigned long long*>(ws);
+  ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * p.nk_stats * 512);
+  mlts_launch_doc_bits(p, bits, st);
+  p.doc_bits = bits;
   return ws;
 }
 
@@ -311,6 +318,43 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
   if (threadIdx.x == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
 }
 
+
+// One block per (batch row, 64-query group), lane = query of the group: walks the key tiles and, for the pairs whose mask
+// the attention kernels evaluate (mixed pairs, and fully visible pairs of a ragged last key tile), forms the 64
+// visibility bits of the lane's query.  Key ids are wave-uniform per step, so they come by scalar loads.
+__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsigned long long* __restrict__ out) {
+  const int g = blockIdx.x % p.nq_stats, b = blockIdx.x / p.nq_stats;
+  const int r = threadIdx.x;
+  const int4 qs = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + g];
+  const int qi = g * kAttnTile + r;
+  int qpos = 0, qseq = -1;
+  if (qi < p.Sq) {
+    qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qi];
+    qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qi];
+  }
+  const int32_t* kpos = p.k_pos + static_cast<int64_t>(b) * p.Sk;
+  const int32_t* kseq = p.k_seq + static_cast<int64_t>(b) * p.Sk;
+  unsigned long long* row = out + (static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats * 64 + r;
+  for (int j = 0; j < p.nk_stats; ++j) {
+    const int4 ks = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
+    int cls = classify_doc_tile(qs, ks);
+    if (cls == TILE_FULL && j * kAttnTile + kAttnTile > p.Sk) cls = TILE_MASKED;
+    if (cls != TILE_MASKED) continue;
+    unsigned long long w = 0;
+    const int n = min(kAttnTile, p.Sk - j * kAttnTile);
+    for (int i = 0; i < n; ++i) {
+      const int kj = j * kAttnTile + i;
+      const bool vis = kpos[kj] <= qpos && kseq[kj] == qseq && qseq >= 0;
+      w |= static_cast<unsigned long long>(vis) << i;
+    }
+    row[static_cast<int64_t>(j) * 64] = w;
+  }
+}
+
+void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, hipStream_t st) {
+  if (p.B * p.nq_stats == 0 || p.nk_stats == 0) return;
+  hipLaunchKernelGGL(doc_bits_kernel, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out);
+}
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
   const int ntiles = (S + kAttnTile - 1) / kAttnTile;

@@ -26,6 +26,11 @@ struct AttnParams {
   const int4* q_stats;  // [B, ceil(Sq/64)] (min_pos, max_pos, min_seq, max_seq)
   const int4* k_stats;  // [B, ceil(Sk/64)]
   int nq_stats, nk_stats;
+  // MLTS_MASK_DOC: for every (64-query group, 64-key tile) pair that classify_doc_tile calls mixed (and for fully visible
+  // pairs of a ragged last key tile), 64 words [B][nq_stats][nk_stats][64]: bit i of word r = key i of the tile is
+  // visible to query r of the group.  The mask is the same for every head and for forward and dQ, so it is evaluated
+  // once per call by a pre-pass instead of per head inside the kernels.  Words of other pairs are not written.
+  const unsigned long long* doc_bits;
   int nqt;              // query tiles per (batch, head) for the launched kernel
 };
 
@@ -130,3 +135,4 @@ __device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);
+void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, hipStream_t st);

@@ -29,8 +29,8 @@ struct FwdCfg {
   static constexpr int CPR = RB / 16;                  // 16-byte chunks per row
   static constexpr int TILE_BYTES = BN * RB;
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES;   // K then V
-  static constexpr int META_OFF = STAGES * STAGE_BYTES;     // document masks: per stage k_pos[64] then k_seq[64], int32
-  static constexpr int META_BYTES = 2 * BN * 4;
+  static constexpr int META_OFF = STAGES * STAGE_BYTES;     // document masks: per stage and wavefront the visibility words
+  static constexpr int META_BYTES = WAVES * 32 * 8;         // of its 32 queries against the stage's 64 keys
   static constexpr int LDS_BYTES = META_OFF + STAGES * META_BYTES;
   static constexpr int PPW = TILE_BYTES / (WAVES * 1024);  // 1 KiB pieces of each tile per wavefront (2 or 1)
   static constexpr int LOADS_PER_TILE = 2 * PPW;           // DMA instructions per wavefront per stage
@@ -176,12 +176,13 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     const int kv0 = j * BN;
     unsigned char* sbase = smem + stage * STAGE_BYTES + wave * PPW * 1024;
     if (MODE == MLTS_MASK_DOC) {
-      // the tile's key positions and sequence ids, for the tiles that need the mask evaluated pair by pair: wavefront w
-      // moves entries 16 w .. 16 w + 15 of (k_pos[64], k_seq[64]) with its first 16 lanes
+      // the visibility words of this wavefront's 32 queries against the tile's keys (256 bytes; read only if the pair is
+      // one whose words the pre-pass wrote, i.e. if the wavefront masks the tile)
       if (lane < 16) {
-        const int e = wave * 16 + lane;
-        const int32_t* src = (e < BN ? p.k_pos : p.k_seq) + static_cast<int64_t>(b) * p.Sk + min(kv0 + (e & (BN - 1)), p.Sk - 1);
-        __builtin_amdgcn_global_load_lds(MLTS_GLB(src), MLTS_LDS(smem + META_OFF + stage * META_BYTES + wave * 64), 4, 0, 0);
+        const int g = min((q0 >> 6) + (wave >> 1), p.nq_stats - 1);
+        const unsigned long long* src =
+            p.doc_bits + ((static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats + j) * 64 + (wave & 1) * 32 + lane * 2;
+        __builtin_amdgcn_global_load_lds(MLTS_GLB(src), MLTS_LDS(smem + META_OFF + stage * META_BYTES + wave * 256), 16, 0, 0);
       }
     }
     if (kv0 + BN <= p.Sk) {
@@ -411,41 +412,26 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
     if (cls != TILE_SKIP) {
       if (cls == TILE_MASKED) {
         if constexpr (MODE == MLTS_MASK_DOC) {
-          // positions and sequence ids of the tile's keys (16 per key block and lane half; groups g = 0..3: keys
-          // kb * 32 + g * 8 + hh * 4 .. + 3) from the stage's copy, all sixteen reads at once: a read issued here waits
-          // out the LDS queue of the other wavefronts' fragment reads, and the second key block's ids travel while the
-          // first block's mask is applied
-          v4i32 kp[2][4], ksq[2][4];
-          const uint32_t ma = lds0 + META_OFF + stage * META_BYTES + (hh * 4) * 4;
+          // this query's visibility bits of the tile's 64 keys (formed once per call by the pre-pass): score register
+          // (kb, g, r) <-> key kb * 32 + g * 8 + hh * 4 + r, so after a shift by hh * 4 the bit positions are constants
+          v2i32 wraw;
+          asm volatile("ds_read_b64 %0, %1" : "=v"(wraw) : "v"(lds0 + META_OFF + stage * META_BYTES + wave * 256 + l32 * 8));
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wraw));
+          const unsigned long long wsh =
+              ((static_cast<unsigned long long>(static_cast<unsigned>(wraw[1])) << 32) | static_cast<unsigned>(wraw[0])) >> (hh * 4);
+          const int wlo = static_cast<int>(wsh), whi = static_cast<int>(wsh >> 32);
+          typedef int i32x16 __attribute__((ext_vector_type(16)));
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb) {
-            kp[kb][0] = kb ? lds_read_b128<128>(ma) : lds_read_b128<0>(ma);
-            kp[kb][1] = kb ? lds_read_b128<160>(ma) : lds_read_b128<32>(ma);
-            kp[kb][2] = kb ? lds_read_b128<192>(ma) : lds_read_b128<64>(ma);
-            kp[kb][3] = kb ? lds_read_b128<224>(ma) : lds_read_b128<96>(ma);
-            ksq[kb][0] = kb ? lds_read_b128<BN * 4 + 128>(ma) : lds_read_b128<BN * 4>(ma);
-            ksq[kb][1] = kb ? lds_read_b128<BN * 4 + 160>(ma) : lds_read_b128<BN * 4 + 32>(ma);
-            ksq[kb][2] = kb ? lds_read_b128<BN * 4 + 192>(ma) : lds_read_b128<BN * 4 + 64>(ma);
-            ksq[kb][3] = kb ? lds_read_b128<BN * 4 + 224>(ma) : lds_read_b128<BN * 4 + 96>(ma);
-          }
+            // whole-vector casts: casting single elements of an MFMA result is miscompiled (element 0 is broadcast)
+            i32x16 si = __builtin_bit_cast(i32x16, sacc[kb]);
 #pragma unroll
-          for (int kb = 0; kb < 2; ++kb) {
-            if (kb == 0) {
-              wait_lgkm<8>(kp[0][0], kp[0][1], kp[0][2], kp[0][3]);
-              wait_lgkm<8>(ksq[0][0], ksq[0][1], ksq[0][2], ksq[0][3]);
-            } else {
-              wait_lgkm<0>(kp[1][0], kp[1][1], kp[1][2], kp[1][3]);
-              wait_lgkm<0>(ksq[1][0], ksq[1][1], ksq[1][2], ksq[1][3]);
+            for (int e = 0; e < 16; ++e) {
+              const int bit = (e >> 2) * 8 + (e & 3);
+              const int keep = __builtin_amdgcn_sbfe(kb ? whi : wlo, bit, 1);  // all ones if visible
+              si[e] = (keep & si[e]) | (~keep & static_cast<int>(0xff800000u));
             }
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const int kbase = kv0 + kb * 32 + g * 8 + hh * 4;
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                const bool vis = (kbase + r < p.Sk) && (kp[kb][g][r] <= qpos) && (ksq[kb][g][r] == qseq) && (qseq >= 0);
-                if (!vis) sacc[kb][g * 4 + r] = -INFINITY;
-              }
-            }
+            sacc[kb] = __builtin_bit_cast(f32x16, si);
           }
         } else {
 #pragma unroll
