@@ -220,13 +220,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     ld_voff[n] = (static_cast<uint32_t>(ld_row[n]) * static_cast<uint32_t>(p.vs[2]) + ld_col[n]) * 2;
   }
   v4i32 stg_k[NLD], stg_v[NLD];
-  int stg_m = 0;  // document masks: threads 0..127 carry the tile's key positions (64) and sequence ids (64)
+  // document masks: this lane's query against the 64 keys of a tile, one bit per key (formed once per call by the pre-pass
+  // for the pairs the kernels mask; other pairs' words are never looked at).  The word of the next tile is fetched with
+  // that tile, always, so that no load of the loop stands under a branch.
+  unsigned long long vis_next = 0;
+  const unsigned long long* vis_row = nullptr;
+  if (MODE == MLTS_MASK_DOC) {
+    const int g = min(wq0 >> 6, p.nq_stats - 1);
+    vis_row = p.doc_bits + (static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats * 64 + ((wq0 >> 5) & 1) * 32 + l32;
+  }
   auto stage_load = [&](int j) {
     const int kv0 = j * BN;
-    if (MODE == MLTS_MASK_DOC && tid < 2 * BN) {
-      const int32_t* src = (tid < BN ? p.k_pos : p.k_seq) + static_cast<int64_t>(b) * p.Sk;
-      stg_m = src[min(kv0 + (tid & (BN - 1)), p.Sk - 1)];
-    }
+    if (MODE == MLTS_MASK_DOC) vis_next = vis_row[static_cast<int64_t>(j) * 64];
     const bf16_t* Kt = K + static_cast<int64_t>(kv0) * p.ks[2];
     const bf16_t* Vt = V + static_cast<int64_t>(kv0) * p.vs[2];
     const int last = p.Sk - 1 - kv0;  // rows past the end repeat the last key; their scores are masked
@@ -251,8 +256,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       lds_write_b128<THREADS * 16>(a, stg_k[NLD - 1]);
       lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_v[NLD - 1]);
     }
-    if (MODE == MLTS_MASK_DOC && tid < 2 * BN)
-      asm volatile("ds_write_b32 %0, %1" ::"v"(lds0 + C::META_OFF + stage * C::META_BYTES + tid * 4), "v"(stg_m));
   };
 
   const int j0 = next_tile(0);
@@ -370,37 +373,33 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   // one 64-key tile for this wavefront's 32 queries, one 32-key block after the other; lane = query, accumulator
   // register e <-> key 32 kb + 8 (e/4) + 4 hh + e%4
-  auto process_tile = [&](const bool masked, const uint32_t so, const int kv0) {
+  auto process_tile = [&](const bool masked, const uint32_t so, const int kv0, const unsigned long long vis) {
     const int klim_t = min(qrow + (MODE == MLTS_MASK_CAUSAL ? p.causal_off : 0x3fffffff), p.Sk - 1) - kv0 - hh * 4;
     bf16x8 dsf[2];
     f32x16 s, dp;
     // masked tiles only (a wave-uniform branch around VALU work, no matrix instruction inside): hidden scores -> -inf
     auto apply_mask = [&](const int kb) {
-      // document masks: positions and sequence ids of the keys come from the stage's copy, four keys at a time (the
-      // registers of a whole block's worth are not to be had at this point of the tile)
-      const uint32_t ma = lds0 + C::META_OFF + (so / STAGE_BYTES) * C::META_BYTES + (kb * 32 + hh * 4) * 4;
+      if constexpr (MODE == MLTS_MASK_DOC) {
+        // register (g, r) <-> key kb * 32 + g * 8 + hh * 4 + r: after a shift by hh * 4 the bit positions are constants
+        typedef int i32x16 __attribute__((ext_vector_type(16)));
+        const unsigned long long wsh = vis >> (hh * 4);
+        const int wbits = static_cast<int>(kb ? wsh >> 32 : wsh);
+        // whole-vector casts: casting single elements of an MFMA result is miscompiled (element 0 is broadcast)
+        i32x16 si = __builtin_bit_cast(i32x16, s);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        if (MODE == MLTS_MASK_DOC) {
-          // positions first, then sequence ids through the same registers
-          v4i32 kp[1];
-          kp[0] = g == 0 ? lds_read_b128<0>(ma) : g == 1 ? lds_read_b128<32>(ma) : g == 2 ? lds_read_b128<64>(ma) : lds_read_b128<96>(ma);
-          wait_lgkm<0>(kp);
+        for (int e = 0; e < 16; ++e) {
+          const int keep = __builtin_amdgcn_sbfe(wbits, (e >> 2) * 8 + (e & 3), 1);  // all ones if visible
+          si[e] = (keep & si[e]) | (~keep & static_cast<int>(0xff800000u));
+        }
+        s = __builtin_bit_cast(f32x16, si);
+      } else {
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (!(kb * 32 + g * 8 + r <= klim_t && kp[0][r] <= qpos && qseq >= 0)) s[g * 4 + r] = -INFINITY;
-          kp[0] = g == 0 ? lds_read_b128<BN * 4>(ma) : g == 1 ? lds_read_b128<BN * 4 + 32>(ma) : g == 2 ? lds_read_b128<BN * 4 + 64>(ma) : lds_read_b128<BN * 4 + 96>(ma);
-          wait_lgkm<0>(kp);
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (kp[0][r] != qseq) s[g * 4 + r] = -INFINITY;
-        } else {
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             // key <= min(query + causal_off, Sk - 1), as one comparison against a per-lane, per-tile threshold
             if (!(kb * 32 + g * 8 + r <= klim_t)) s[g * 4 + r] = -INFINITY;
           }
-        }
       }
     };
     auto ds_block = [&](const int kb) {
@@ -483,6 +482,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       const int doc_cls = MODE == MLTS_MASK_DOC ? doc_scan_class(scan, j) : TILE_FULL;  // before the scan moves on
       const int jn = next_tile(j + 1);
       drain_and_barrier();
+      const unsigned long long vis = vis_next;  // of tile j; stage_load fetches the next tile's
       if (jn < j_end) stage_load(jn);
 
       const int kv0 = j * BN;
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       }
       if (cls == TILE_FULL && kv0 + BN > p.Sk) cls = TILE_MASKED;  // ragged last tile: key < Sk
       if (wq0 >= p.Sq) cls = TILE_SKIP;
-      if (cls != TILE_SKIP) process_tile(cls == TILE_MASKED, stage * STAGE_BYTES, kv0);
+      if (cls != TILE_SKIP) process_tile(cls == TILE_MASKED, stage * STAGE_BYTES, kv0, vis);
 
       if (jn < j_end) stage_store(stage ^ 1);
       j = jn;
