@@ -49,12 +49,12 @@ const char* shape_problem(const mlts_attn_shape* s) {
   return nullptr;
 }
 
-int64_t stats_bytes(const mlts_attn_shape* s) {
+int64_t stats_bytes(const mlts_attn_shape* s, bool backward) {
   if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return 0;
   const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
   // tile statistics of both sides, then the visibility bits of the mixed (query group, key tile) pairs (512 bytes per
-  // pair, indexed densely: Sq * Sk / 8 bytes per batch row)
-  return align256(s->B * nq * 16) + align256(s->B * nk * 16) + align256(s->B * nq * nk * 512);
+  // pair, indexed densely: Sq * Sk / 8 bytes per batch row), query-major and, for the backward pass, key-major as well
+  return align256(s->B * nq * 16) + align256(s->B * nk * 16) + (backward ? 2 : 1) * align256(s->B * nq * nk * 512);
 }
 
 void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o,
@@ -85,14 +85,15 @@ void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const v
   p.q_stats = nullptr;
   p.k_stats = nullptr;
   p.doc_bits = nullptr;
+  p.doc_bits_k = nullptr;
   p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
   p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
   p.nqt = 0;
 }
 
 // Carves the tile statistics out of the front of the workspace and launches their kernels.
-char* setup_stats(AttnParams& p, const mlts_attn_shape* s, char* ws, hipStream_t st) {
-  if (stats_bytes(s) == 0) return ws;
+char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* ws, hipStream_t st) {
+  if (stats_bytes(s, backward) == 0) return ws;
   int4* qst = reinterpret_cast<int4*>(ws);
   ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * 16);
   int4* kst = reinterpret_cast<int4*>(ws);
@@ -103,8 +104,14 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, char* ws, hipStream_t
   p.k_stats = kst;
   unsigned long long* bits = reinterpret_cast<unsigned long long*>(ws);
   ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * p.nk_stats * 512);
-  mlts_launch_doc_bits(p, bits, st);
+  unsigned long long* bits_k = nullptr;
+  if (backward) {
+    bits_k = reinterpret_cast<unsigned long long*>(ws);
+    ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * p.nk_stats * 512);
+  }
+  mlts_launch_doc_bits(p, bits, bits_k, st);
   p.doc_bits = bits;
+  p.doc_bits_k = bits_k;
   return ws;
 }
 
@@ -180,7 +187,7 @@ int64_t ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32) {
 int64_t bwd_min_workspace(const mlts_attn_shape* s) {
   const int64_t delta = align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
   const int64_t lse2 = uses_mfma(s) ? mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq) : 0;
-  return stats_bytes(s) + delta + lse2;
+  return stats_bytes(s, true) + delta + lse2;
 }
 
 // Default: the recomputing dQ kernel first, which also writes the row statistics (delta, lse2) into the workspace, then
@@ -218,7 +225,7 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
                (long long)workspace_bytes, (long long)need);
   AttnBwdParams bp;
   fill_params(bp.a, s, q, k, v, const_cast<void*>(o), const_cast<float*>(lse));
-  char* ws = setup_stats(bp.a, s, static_cast<char*>(workspace), st);
+  char* ws = setup_stats(bp.a, s, true, static_cast<char*>(workspace), st);
   float* delta = reinterpret_cast<float*>(ws);
   ws += align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
   bp.dout = dout;
@@ -321,8 +328,11 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
 
 // One block per (batch row, 64-query group), lane = query of the group: walks the key tiles and, for the pairs whose mask
 // the attention kernels evaluate (mixed pairs, and fully visible pairs of a ragged last key tile), forms the 64
-// visibility bits of the lane's query.  Key ids are wave-uniform per step, so they come by scalar loads.
-__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsigned long long* __restrict__ out) {
+// visibility bits of the lane's query.  Key ids are wave-uniform per step, so they come by scalar loads.  The ballot of
+// one step is the key-major word of that key (which queries of the group see it); lane i keeps the one of key i.
+template <bool KEY_MAJOR>
+__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsigned long long* __restrict__ out,
+                                                      unsigned long long* __restrict__ out_k) {
   const int g = blockIdx.x % p.nq_stats, b = blockIdx.x / p.nq_stats;
   const int r = threadIdx.x;
   const int4 qs = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + g];
@@ -340,20 +350,26 @@ __global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsign
     int cls = classify_doc_tile(qs, ks);
     if (cls == TILE_FULL && j * kAttnTile + kAttnTile > p.Sk) cls = TILE_MASKED;
     if (cls != TILE_MASKED) continue;
-    unsigned long long w = 0;
+    unsigned long long w = 0, wk = 0;
     const int n = min(kAttnTile, p.Sk - j * kAttnTile);
     for (int i = 0; i < n; ++i) {
       const int kj = j * kAttnTile + i;
       const bool vis = kpos[kj] <= qpos && kseq[kj] == qseq && qseq >= 0;
       w |= static_cast<unsigned long long>(vis) << i;
+      if (KEY_MAJOR) {
+        const unsigned long long col = __builtin_amdgcn_ballot_w64(vis);
+        if (r == i) wk = col;
+      }
     }
     row[static_cast<int64_t>(j) * 64] = w;
+    if (KEY_MAJOR) out_k[((static_cast<int64_t>(b) * p.nk_stats + j) * p.nq_stats + g) * 64 + r] = wk;
   }
 }
 
-void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, hipStream_t st) {
+void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st) {
   if (p.B * p.nq_stats == 0 || p.nk_stats == 0) return;
-  hipLaunchKernelGGL(doc_bits_kernel, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out);
+  if (out_k) hipLaunchKernelGGL(doc_bits_kernel<true>, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out, out_k);
+  else hipLaunchKernelGGL(doc_bits_kernel<false>, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out, out_k);
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
@@ -366,7 +382,7 @@ extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return sha
 
 extern "C" int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s) {
   if (shape_problem(s)) return -1;
-  return stats_bytes(s);
+  return stats_bytes(s, false);
 }
 
 extern "C" int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32) {
@@ -387,7 +403,7 @@ extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void
   if (s->B == 0 || s->Sq == 0) return MLTS_OK;
   MLTS_REQUIRE(q && o && lse, "mlts_attn_fwd: q, o, lse must be non-null");
   MLTS_REQUIRE(s->Sk == 0 || (k && v), "mlts_attn_fwd: k, v must be non-null");
-  const int64_t need = stats_bytes(s);
+  const int64_t need = stats_bytes(s, false);
   MLTS_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), "mlts_attn_fwd: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)need);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -396,7 +412,7 @@ extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void
   if (uses_mfma(s)) {
     MLTS_REQUIRE(mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) && mlts_aligned16(o),
                  "mlts_attn_fwd: q, k, v, o must be 16-byte aligned");
-    setup_stats(p, s, static_cast<char*>(workspace), st);
+    setup_stats(p, s, false, static_cast<char*>(workspace), st);
     return mlts_attn_fwd_bf16_dma(p, s->D, s->mask_mode, st);
   }
   return mlts_attn_generic_fwd(p, s->D, s->dtype, s->mask_mode, st);

@@ -167,11 +167,12 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     }
   }
   const int4 wk_stats = MODE == MLTS_MASK_DOC ? ((kb >> 1) ? kstats[1] : kstats[0]) : make_int4(0, 0, 0, 0);
-  int kpos = 0, kseq = -2;
-  if (MODE == MLTS_MASK_DOC && kj < p.Sk) {
-    kpos = p.k_pos[static_cast<int64_t>(b) * p.Sk + kj];
-    kseq = p.k_seq[static_cast<int64_t>(b) * p.Sk + kj];
-  }
+  // document masks: the lane's key has one 64-bit word per query tile (bit i = query i of the tile sees the key),
+  // formed by a pre-pass for the tiles that classify() calls masked; role 0 fetches it along with the tile
+  const unsigned long long* vis_row = nullptr;
+  unsigned long long vis_next = 0;
+  if (MODE == MLTS_MASK_DOC)
+    vis_row = p.doc_bits_k + (static_cast<int64_t>(b) * p.nk_stats + min(wkv0 >> 6, p.nk_stats - 1)) * p.nq_stats * 64 + (wkv0 & 32) + l32;
   // The walk over (query head of the group, query tile) is kept as two counters; a position past the end has
   // h == group.  (No division by the runtime tile count in the loop.)
   struct Pos {
@@ -212,7 +213,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     } else if (MODE == MLTS_MASK_DOC) {
       cls = doc_scan_class(scan, x.qt);
     }
-    if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || q0 + BQ > p.Sq)) cls = TILE_MASKED;
+    // (with a document mask, queries past Sq need no mask: their lse2 is +inf)
+    if (cls == TILE_FULL && (wkv0 + 32 > p.Sk || (MODE != MLTS_MASK_DOC && q0 + BQ > p.Sq))) cls = TILE_MASKED;
     if (wkv0 >= p.Sk) cls = TILE_SKIP;
     return cls;
   };
@@ -260,14 +262,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       const int64_t srow = (static_cast<int64_t>(b) * p.Hq + hq) * p.Sq;
       const int r = q0 + (tid & (BQ - 1));
       stg_s = tid < BQ ? lse2[r < p.Sq ? srow + r : lse2_inf] : bp.delta[srow + min(r, p.Sq - 1)];
-    } else if (MODE == MLTS_MASK_DOC && tid < 4 * BQ) {
-      // the tile's query positions and sequence ids (as raw bits), for the tiles whose mask is evaluated pair by pair;
-      // rows past the end are padding
-      const int r = q0 + (tid & (BQ - 1));
-      const int32_t* src = (tid < 3 * BQ ? p.q_pos : p.q_seq) + static_cast<int64_t>(b) * p.Sq;
-      const int v = r < p.Sq ? src[r] : (tid < 3 * BQ ? -0x7fffffff : -1);
-      stg_s = __builtin_bit_cast(float, v);
     }
+    if (MODE == MLTS_MASK_DOC && role == 0) vis_next = vis_row[static_cast<int64_t>(qt_begin + x.qt) * 64];
   };
   const uint32_t stg_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(MLTS_LDS(smem))) + tid * 16;
   auto stage_store = [&](int stage) {
@@ -278,7 +274,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       lds_write_b128<THREADS * 16>(a, stg_q[NLD - 1]);
       lds_write_b128<TILE_BYTES + THREADS * 16>(a, stg_d[NLD - 1]);
     }
-    if (tid < (MODE == MLTS_MASK_DOC ? 4 : 2) * BQ)
+    if (tid < 2 * BQ)
       asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(lds0_ + stage * STAGE_BYTES + tid * 4), "v"(stg_s), "n"(STAT_OFF));
   };
 
@@ -361,7 +357,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       (u / DB) ? AFRAG1 : AFRAG0, as_frag(src[2 * u], src[2 * u + 1]), acc[u % DB], 0, 0, 0);
 
   // ---- role 0: one tile.  lane = key, accumulator register e <-> query 32 qb + 8 (e/4) + 4 hh + e%4 ----
-  auto role0_tile = [&](const bool masked, const int q0, const int stage, const int pbuf) {
+  auto role0_tile = [&](const bool masked, const int q0, const int stage, const int pbuf, const unsigned long long vis) {
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
     uint32_t ra[KS];
 #pragma unroll
@@ -380,27 +376,29 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       constexpr int qb = decltype(qb_tag)::value;
       // the comparisons below belong to masked tiles only: an opaque copy of their operand keeps the compiler from
       // hoisting all of them in front of the wave-uniform branch, where every tile would pay for them
-      int causal_here = causal_t;
-      asm volatile("" : "+v"(causal_here));
-      // document masks: positions and sequence ids of the queries come from the stage, four queries at a time
-      const uint32_t ma = sb + STAT_OFF + 2 * BQ * 4 + (qb * 32 + hh * 4) * 4;
+      if constexpr (MODE == MLTS_MASK_DOC) {
+        // bit 32 qb + 8 g + 4 hh + r of the key's word; the scores are handled as one integer vector (a cast of a
+        // single element of a matrix result is miscompiled)
+        typedef int i32x16 __attribute__((ext_vector_type(16)));
+        const unsigned long long wsh = vis >> (hh * 4);
+        const int wbits = static_cast<int>(qb ? (wsh >> 32) : wsh);
+        i32x16 si = __builtin_bit_cast(i32x16, s);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        v4i32 qm[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [0] positions, [1] sequence ids of queries qb * 32 + g * 8 + hh * 4 .. + 3
-        if (MODE == MLTS_MASK_DOC) {
-          qm[0] = g == 0 ? lds_read_b128<0>(ma) : g == 1 ? lds_read_b128<32>(ma) : g == 2 ? lds_read_b128<64>(ma) : lds_read_b128<96>(ma);
-          qm[1] = g == 0 ? lds_read_b128<BQ * 4>(ma) : g == 1 ? lds_read_b128<BQ * 4 + 32>(ma) : g == 2 ? lds_read_b128<BQ * 4 + 64>(ma) : lds_read_b128<BQ * 4 + 96>(ma);
-          wait_lgkm<0>(qm);
+        for (int e = 0; e < 16; ++e) {
+          const int keep = __builtin_amdgcn_sbfe(wbits, (e >> 2) * 8 + (e & 3), 1);  // 0 or -1
+          si[e] = (keep & si[e]) | (~keep & static_cast<int>(0xff800000u));
         }
+        s = __builtin_bit_cast(f32x16, si);
+      } else {
+        int causal_here = causal_t;
+        asm volatile("" : "+v"(causal_here));
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          bool vis;
-          if (MODE == MLTS_MASK_CAUSAL) {
-            vis = causal_here <= qb * 32 + g * 8 + r;  // key <= query + causal_off; rows past Sq already give p = 0
-          } else {
-            vis = kj < p.Sk && (kpos <= qm[0][r]) && (kseq == qm[1][r]) && (qm[1][r] >= 0);
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            // key <= query + causal_off; rows past Sq already give p = 0
+            if (!(causal_here <= qb * 32 + g * 8 + r)) s[g * 4 + r] = -INFINITY;
           }
-          if (!vis) s[g * 4 + r] = -INFINITY;
         }
       }
     };
@@ -672,6 +670,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     Pos prev_it = it;
     while (!at_end(it)) {
       const int cls = classify(it);  // before the scan of the needed tiles moves on
+      const unsigned long long vis = vis_next;
       Pos itn = it;
       step(itn);
       itn = first_needed(itn);
@@ -683,7 +682,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         // one instance of the tile body (with several, the register allocator keeps the accumulators twice); the
         // mask is a branch around VALU work inside it.  Without a mask mode nothing needs masking: keys past Sk are
         // never stored and queries past Sq have lse2 = +inf.
-        if (cls != TILE_SKIP) role0_tile(MODE != MLTS_MASK_NONE && cls == TILE_MASKED, q0, stage, pbuf);
+        if (cls != TILE_SKIP) role0_tile(MODE != MLTS_MASK_NONE && cls == TILE_MASKED, q0, stage, pbuf, vis);
       } else {
         if (prev_active) role1_ds(pbuf ^ (4 * PBUF_BYTES));
         if (cls != TILE_SKIP) role1_dp(stage);

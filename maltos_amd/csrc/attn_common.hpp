@@ -31,6 +31,9 @@ struct AttnParams {
   // visible to query r of the group.  The mask is the same for every head and for forward and dQ, so it is evaluated
   // once per call by a pre-pass instead of per head inside the kernels.  Words of other pairs are not written.
   const unsigned long long* doc_bits;
+  // The same bits for the mixed pairs, key-major, for the dK/dV kernel whose lanes are keys: [B][nk_stats][nq_stats][64],
+  // bit i of word r = query i of the group sees key r of the tile.  Null in the forward pass.
+  const unsigned long long* doc_bits_k;
   int nqt;              // query tiles per (batch, head) for the launched kernel
 };
 
@@ -135,4 +138,4 @@ __device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);
-void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, hipStream_t st);
+void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st);
