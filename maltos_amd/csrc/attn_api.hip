@@ -326,16 +326,30 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
 }
 
 
-// One block per (batch row, 64-query group), lane = query of the group: walks the key tiles and, for the pairs whose mask
-// the attention kernels evaluate (mixed pairs, and fully visible pairs of a ragged last key tile), forms the 64
-// visibility bits of the lane's query.  Key ids are wave-uniform per step, so they come by scalar loads.  The ballot of
-// one step is the key-major word of that key (which queries of the group see it); lane i keeps the one of key i.
+// One wavefront per (batch row, 64-query group, kDocBitsChunk key tiles), lane = query of the group.  For each pair of
+// the chunk whose mask the attention kernels evaluate (mixed pairs, and fully visible pairs of a ragged last key tile)
+// the lanes load one key's ids each and the 64 keys are walked with lane reads: a pair costs one memory round trip
+// and a few hundred instructions, and a query group that straddles a document boundary (every key tile of both
+// documents is mixed for it) is spread over many wavefronts.  The ballot of one step is the key-major word of that key
+// (which queries of the group see it); it goes into lane i of the key-major result.
+constexpr int kDocBitsChunk = 4;
+
 template <bool KEY_MAJOR>
-__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsigned long long* __restrict__ out,
+__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, int n_chunks, unsigned long long* __restrict__ out,
                                                       unsigned long long* __restrict__ out_k) {
-  const int g = blockIdx.x % p.nq_stats, b = blockIdx.x / p.nq_stats;
+  const int chunk = blockIdx.x % n_chunks, bg = blockIdx.x / n_chunks;
+  const int g = bg % p.nq_stats, b = bg / p.nq_stats;
   const int r = threadIdx.x;
   const int4 qs = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + g];
+  const int t = chunk * kDocBitsChunk + r;  // lane r < kDocBitsChunk classifies key tile t
+  bool mixed = false;
+  if (r < kDocBitsChunk && t < p.nk_stats) {
+    const int4 ks = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + t];
+    const int cls = classify_doc_tile(qs, ks);
+    mixed = cls == TILE_MASKED || (cls == TILE_FULL && t * kAttnTile + kAttnTile > p.Sk);
+  }
+  unsigned long long todo = __builtin_amdgcn_ballot_w64(mixed);
+  if (todo == 0) return;
   const int qi = g * kAttnTile + r;
   int qpos = 0, qseq = -1;
   if (qi < p.Sq) {
@@ -344,37 +358,55 @@ __global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, unsign
   }
   const int32_t* kpos = p.k_pos + static_cast<int64_t>(b) * p.Sk;
   const int32_t* kseq = p.k_seq + static_cast<int64_t>(b) * p.Sk;
-  unsigned long long* row = out + (static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats * 64 + r;
-  for (int j = 0; j < p.nk_stats; ++j) {
-    const int4 ks = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + j];
-    int cls = classify_doc_tile(qs, ks);
-    if (cls == TILE_FULL && j * kAttnTile + kAttnTile > p.Sk) cls = TILE_MASKED;
-    if (cls != TILE_MASKED) continue;
-    unsigned long long w = 0, wk = 0;
-    const int n = min(kAttnTile, p.Sk - j * kAttnTile);
-    for (int i = 0; i < n; ++i) {
-      const int kj = j * kAttnTile + i;
-      const bool vis = kpos[kj] <= qpos && kseq[kj] == qseq && qseq >= 0;
+  // the ids of every tile of the chunk are requested before the first pair is walked (one memory latency per wavefront)
+  int kp[kDocBitsChunk], ksq[kDocBitsChunk];
+#pragma unroll
+  for (int c = 0; c < kDocBitsChunk; ++c) {
+    const int kj = (chunk * kDocBitsChunk + c) * kAttnTile + r;
+    kp[c] = 0;
+    ksq[c] = -2;  // keys past the end: an id that no query has
+    if (((todo >> c) & 1ull) && kj < p.Sk) {
+      kp[c] = kpos[kj];
+      ksq[c] = kseq[kj];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kDocBitsChunk; ++c) {
+    if (!((todo >> c) & 1ull)) continue;
+    const int j = chunk * kDocBitsChunk + c;
+    unsigned long long w = 0;
+    int wk_lo = 0, wk_hi = 0;
+#pragma unroll
+    for (int i = 0; i < kAttnTile; ++i) {
+      const int kpi = __builtin_amdgcn_readlane(kp[c], i), ksi = __builtin_amdgcn_readlane(ksq[c], i);
+      const bool vis = kpi <= qpos && ksi == qseq && qseq >= 0;
       w |= static_cast<unsigned long long>(vis) << i;
       if (KEY_MAJOR) {
         const unsigned long long col = __builtin_amdgcn_ballot_w64(vis);
-        if (r == i) wk = col;
+        asm("v_writelane_b32 %0, %1, %2" : "+v"(wk_lo) : "s"(static_cast<int>(col)), "n"(i));
+        asm("v_writelane_b32 %0, %1, %2" : "+v"(wk_hi) : "s"(static_cast<int>(col >> 32)), "n"(i));
       }
     }
-    row[static_cast<int64_t>(j) * 64] = w;
-    if (KEY_MAJOR) out_k[((static_cast<int64_t>(b) * p.nk_stats + j) * p.nq_stats + g) * 64 + r] = wk;
+    out[((static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats + j) * 64 + r] = w;
+    if (KEY_MAJOR)
+      out_k[((static_cast<int64_t>(b) * p.nk_stats + j) * p.nq_stats + g) * 64 + r] =
+          (static_cast<unsigned long long>(static_cast<unsigned>(wk_hi)) << 32) | static_cast<unsigned>(wk_lo);
   }
 }
 
 void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st) {
   if (p.B * p.nq_stats == 0 || p.nk_stats == 0) return;
-  if (out_k) hipLaunchKernelGGL(doc_bits_kernel<true>, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out, out_k);
-  else hipLaunchKernelGGL(doc_bits_kernel<false>, dim3(p.B * p.nq_stats), dim3(64), 0, st, p, out, out_k);
+  const int n_chunks = (p.nk_stats + kDocBitsChunk - 1) / kDocBitsChunk;
+  const int64_t blocks = static_cast<int64_t>(p.B) * p.nq_stats * n_chunks;
+  MltsKernelTimer timer("attn_doc_bits", st);
+  if (out_k) hipLaunchKernelGGL(doc_bits_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
+  else hipLaunchKernelGGL(doc_bits_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
   const int ntiles = (S + kAttnTile - 1) / kAttnTile;
   if (B * ntiles == 0) return;
+  MltsKernelTimer timer("attn_tile_stats", st);
   hipLaunchKernelGGL(tile_stats_kernel, dim3(B * ntiles), dim3(64), 0, st, pos, seq, S, ntiles, out);
 }
 
