@@ -75,13 +75,13 @@ def timed(torch, fn, steps, warmup):
     """Mean seconds per call.  The interpreter's cyclic garbage collector is held off during the timed calls (as
     timeit does): one full collection is a 50-100 ms pause, which in a launch-bound loop of ten steps is the result."""
     import gc
-    preheat(torch, fn)
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    gc.collect()
+    gc.collect()  # before the pre-heat: a collection behind it would leave the GPU idle long enough to drop its clocks
     gc.disable()
     try:
+        preheat(torch, fn)
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             fn()
@@ -189,7 +189,8 @@ def bench_cfg3_packed_gqa(torch, ops, _lib, dev, steps, warmup):
     k = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
     v = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
     do = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
-    ids = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+    # int32 ids, as the C-ABI takes them: converted once per batch (every layer's attention shares them), not per call
+    ids = dict(q_pos=pos.int().to(dev), k_pos=pos.int().to(dev), q_seq=seq.int().to(dev), k_seq=seq.int().to(dev))
 
     def step():
         o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, **ids)

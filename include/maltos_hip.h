@@ -82,8 +82,10 @@ typedef struct mlts_attn_shape {
 const char* mlts_attn_supports(const mlts_attn_shape* s);
 
 /* Bytes of device workspace mlts_attn_fwd / mlts_attn_bwd need for this shape: the per-row statistics the kernels
- * share (delta, LSE in base 2) and, with MLTS_MASK_DOC, the per-tile position / sequence-id ranges.  O(B * Hq * Sq),
- * the workspace class of the flash backward the reference calls (runtime/layers/flash_utils.py:239-258). */
+ * share (delta, LSE in base 2): O(B * Hq * Sq), the workspace class of the flash backward the reference calls
+ * (runtime/layers/flash_utils.py:239-258).  With MLTS_MASK_DOC also the per-tile position / sequence-id ranges and
+ * the visibility bits of the (64 queries, 64 keys) pairs that a document boundary or the causal diagonal cuts, which a
+ * pre-pass forms once per call for all heads: B * Sq * Sk / 8 bytes (forward), twice that (backward). */
 int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s);
 int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32);
 
@@ -117,8 +119,8 @@ int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_s
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
  * results as mlts_attn_bwd with a workspace of exactly mlts_attn_bwd_workspace_bytes (the recomputing backward); the
  * workspace is a buffer of MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE bytes inside the library image, one copy per GPU, held
- * until the process ends.  Shapes whose workspace is larger (about B * Hq * Sq > 1 M query rows) are rejected with
- * MLTS_ERR_INVALID.  No hipMalloc / hipFree is made.  All calls on one GPU share that buffer: calls that may overlap
+ * until the process ends.  Shapes whose workspace is larger (about B * Hq * Sq > 1 M query rows; with MLTS_MASK_DOC
+ * also B * Sq * Sk / 4 bytes of visibility bits, e.g. B * S * S beyond about 28 M) are rejected with MLTS_ERR_INVALID.  No hipMalloc / hipFree is made.  All calls on one GPU share that buffer: calls that may overlap
  * on one GPU (different streams, different threads) race; serialise them or use mlts_attn_bwd. */
 #define MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE (8 << 20)
 int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,

@@ -36,7 +36,7 @@ struct SplitCfg {
   static constexpr int RB = D * 2;                   // bytes per tile row
   static constexpr int CPR = RB / 16;                // 16-byte chunks per row
   static constexpr int TILE_BYTES = BQ * RB;
-  static constexpr int STAT_OFF = 2 * TILE_BYTES;    // lse2[64], delta[64] (fp32), then q_pos[64], q_seq[64] (int32, document masks)
+  static constexpr int STAT_OFF = 2 * TILE_BYTES;    // lse2[64], delta[64] (fp32); the rest of the stage's last KiB is unused
   static constexpr int STAGE_BYTES = STAT_OFF + 4 * BQ * 4;
   static constexpr int PBUF_OFF = STAGES * STAGE_BYTES;
   static constexpr int LDS_BYTES = PBUF_OFF + 2 * 4 * PBUF_BYTES;
