@@ -54,7 +54,9 @@ int64_t stats_bytes(const mlts_attn_shape* s, bool backward) {
   const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
   // tile statistics of both sides, then the visibility bits of the mixed (query group, key tile) pairs (512 bytes per
   // pair, indexed densely: Sq * Sk / 8 bytes per batch row), query-major and, for the backward pass, key-major as well
-  return align256(s->B * nq * 16) + align256(s->B * nk * 16) + (backward ? 2 : 1) * align256(s->B * nq * nk * 512);
+  int64_t n = align256(s->B * nq * 16) + align256(s->B * nk * 16) + (backward ? 2 : 1) * align256(s->B * nq * nk * 512);
+  if (backward) n += 2 * align256(s->B * ((s->Sk + 127) / 128) * 4);  // work count and order of the 128-key blocks
+  return n;
 }
 
 void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o,
@@ -86,6 +88,7 @@ void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const v
   p.k_stats = nullptr;
   p.doc_bits = nullptr;
   p.doc_bits_k = nullptr;
+  p.kblock_order = nullptr;
   p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
   p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
   p.nqt = 0;
@@ -112,6 +115,17 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* 
   mlts_launch_doc_bits(p, bits, bits_k, st);
   p.doc_bits = bits;
   p.doc_bits_k = bits_k;
+  if (backward) {
+    const int64_t n_blocks = static_cast<int64_t>(s->B) * ((s->Sk + 127) / 128);
+    int* work = reinterpret_cast<int*>(ws);
+    ws += align256(n_blocks * 4);
+    int* order = reinterpret_cast<int*>(ws);
+    ws += align256(n_blocks * 4);
+    if (n_blocks > 1 && n_blocks <= kMaxOrderedBlocks) {
+      mlts_launch_kblock_order(p, work, order, st);
+      p.kblock_order = order;
+    }
+  }
   return ws;
 }
 
@@ -401,6 +415,55 @@ void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned
   MltsKernelTimer timer("attn_doc_bits", st);
   if (out_k) hipLaunchKernelGGL(doc_bits_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
   else hipLaunchKernelGGL(doc_bits_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
+}
+
+// Number of query tiles that 128-key block kt of batch row b needs (entry kt * B + b): the same test as the dK/dV kernel's
+// scan of the query statistics.  One wavefront per block.
+__global__ __launch_bounds__(64) void doc_kblock_work_kernel(const AttnParams p, int* __restrict__ work) {
+  const int e = blockIdx.x, b = e % p.B, kt = e / p.B, lane = threadIdx.x;
+  int4 ks[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int t = kt * 2 + i;
+    ks[i] = t < p.nk_stats ? p.k_stats[static_cast<int64_t>(b) * p.nk_stats + t] : make_int4(0x7fffffff, 0, 0, -2);
+  }
+  int cnt = 0;
+  for (int base = 0; base < p.nq_stats; base += 64) {
+    bool need = false;
+    if (base + lane < p.nq_stats) {
+      const int4 qs = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + base + lane];
+      need = classify_doc_tile(qs, ks[0]) != TILE_SKIP || classify_doc_tile(qs, ks[1]) != TILE_SKIP;
+    }
+    cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(need));
+  }
+  if (lane == 0) work[e] = cnt;
+}
+
+// order[rank of i] = i, ranks by work descending (ties by index): every thread counts the entries in front of its own
+__global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ work, int n, int* __restrict__ order) {
+  __shared__ int chunk[256];
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int wi = i < n ? work[i] : 0;
+  int rank = 0;
+  for (int base = 0; base < n; base += 256) {
+    __syncthreads();
+    chunk[threadIdx.x] = base + threadIdx.x < n ? work[base + threadIdx.x] : -1;
+    __syncthreads();
+    const int m = min(256, n - base);
+    for (int j = 0; j < m; ++j) {
+      const int wj = chunk[j];
+      rank += (wj > wi || (wj == wi && base + j < i)) ? 1 : 0;
+    }
+  }
+  if (i < n) order[rank] = i;
+}
+
+void mlts_launch_kblock_order(const AttnParams& p, int* work, int* order, hipStream_t st) {
+  const int n = p.B * ((p.Sk + 127) / 128);
+  if (n == 0) return;
+  MltsKernelTimer timer("attn_doc_order", st);
+  hipLaunchKernelGGL(doc_kblock_work_kernel, dim3(n), dim3(64), 0, st, p, work);
+  hipLaunchKernelGGL(doc_order_kernel, dim3((n + 255) / 256), dim3(256), 0, st, work, n, order);
 }
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {

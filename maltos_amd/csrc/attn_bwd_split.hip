@@ -128,9 +128,18 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
 
   const int nbh = p.B * p.Hkv;
   const int bid = blockIdx.x;
-  const int kt = bid / nbh;  // key tile; low tiles see the most queries under a causal mask and go first
+  int kt = bid / nbh;  // key tile; low tiles see the most queries under a causal mask and go first
   const int bh = bid % nbh;
-  const int b = bh / p.Hkv, hkv = bh % p.Hkv;
+  int b = bh / p.Hkv;
+  const int hkv = bh % p.Hkv;
+  if constexpr (MODE == MLTS_MASK_DOC) {
+    // document masks: the (key tile, batch row) pairs are walked in the order of their work, most first
+    if (p.kblock_order) {
+      const int e = p.kblock_order[kt * p.B + b];
+      kt = e / p.B;
+      b = e % p.B;
+    }
+  }
   const int group = p.Hq / p.Hkv;
   const int kv0 = kt * BKV;
   const int wkv0 = kv0 + kb * 32;

@@ -34,6 +34,11 @@ struct AttnParams {
   // The same bits for the mixed pairs, key-major, for the dK/dV kernel whose lanes are keys: [B][nk_stats][nq_stats][64],
   // bit i of word r = query i of the group sees key r of the tile.  Null in the forward pass.
   const unsigned long long* doc_bits_k;
+  // Backward with MLTS_MASK_DOC: the (128-key block, batch row) pairs, index kt * B + b, sorted by the number of query
+  // tiles they need, most first.  The dK/dV grid walks them in this order: a block's work ranges from one tile to all
+  // tiles of two long documents, and in plain order a heavy block that starts late sets the kernel's duration.  Null:
+  // plain order.
+  const int* kblock_order;
   int nqt;              // query tiles per (batch, head) for the launched kernel
 };
 
@@ -139,3 +144,6 @@ __device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
 
 void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);
 void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st);
+// order[0 .. B * nkt) for AttnParams::kblock_order (nkt = 128-key blocks per row); work: B * nkt ints of scratch
+constexpr int kMaxOrderedBlocks = 8192;
+void mlts_launch_kblock_order(const AttnParams& p, int* work, int* order, hipStream_t st);
