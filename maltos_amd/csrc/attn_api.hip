@@ -55,7 +55,8 @@ int64_t stats_bytes(const mlts_attn_shape* s, bool backward) {
   // tile statistics of both sides, then the visibility bits of the mixed (query group, key tile) pairs (512 bytes per
   // pair, indexed densely: Sq * Sk / 8 bytes per batch row), query-major and, for the backward pass, key-major as well
   int64_t n = align256(s->B * nq * 16) + align256(s->B * nk * 16) + (backward ? 2 : 1) * align256(s->B * nq * nk * 512);
-  if (backward) n += 2 * align256(s->B * ((s->Sk + 127) / 128) * 4);  // work count and order of the 128-key blocks
+  n += 2 * align256(s->B * nq * 4);                                   // work count and order of the query blocks
+  if (backward) n += 2 * align256(s->B * ((s->Sk + 127) / 128) * 4);  // ... and of the 128-key blocks
   return n;
 }
 
@@ -89,45 +90,14 @@ void fill_params(AttnParams& p, const mlts_attn_shape* s, const void* q, const v
   p.doc_bits = nullptr;
   p.doc_bits_k = nullptr;
   p.kblock_order = nullptr;
+  p.qblock_order = nullptr;
   p.nq_stats = (s->Sq + kAttnTile - 1) / kAttnTile;
   p.nk_stats = (s->Sk + kAttnTile - 1) / kAttnTile;
   p.nqt = 0;
+  p.head_pack_shift = 0;
 }
 
-// Carves the tile statistics out of the front of the workspace and launches their kernels.
-char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* ws, hipStream_t st) {
-  if (stats_bytes(s, backward) == 0) return ws;
-  int4* qst = reinterpret_cast<int4*>(ws);
-  ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * 16);
-  int4* kst = reinterpret_cast<int4*>(ws);
-  ws += align256(static_cast<int64_t>(s->B) * p.nk_stats * 16);
-  mlts_launch_tile_stats(s->q_pos, s->q_seq, s->B, s->Sq, qst, st);
-  mlts_launch_tile_stats(s->k_pos, s->k_seq, s->B, s->Sk, kst, st);
-  p.q_stats = qst;
-  p.k_stats = kst;
-  unsigned long long* bits = reinterpret_cast<unsigned long long*>(ws);
-  ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * p.nk_stats * 512);
-  unsigned long long* bits_k = nullptr;
-  if (backward) {
-    bits_k = reinterpret_cast<unsigned long long*>(ws);
-    ws += align256(static_cast<int64_t>(s->B) * p.nq_stats * p.nk_stats * 512);
-  }
-  mlts_launch_doc_bits(p, bits, bits_k, st);
-  p.doc_bits = bits;
-  p.doc_bits_k = bits_k;
-  if (backward) {
-    const int64_t n_blocks = static_cast<int64_t>(s->B) * ((s->Sk + 127) / 128);
-    int* work = reinterpret_cast<int*>(ws);
-    ws += align256(n_blocks * 4);
-    int* order = reinterpret_cast<int*>(ws);
-    ws += align256(n_blocks * 4);
-    if (n_blocks > 1 && n_blocks <= kMaxOrderedBlocks) {
-      mlts_launch_kblock_order(p, work, order, st);
-      p.kblock_order = order;
-    }
-  }
-  return ws;
-}
+char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* ws, hipStream_t st);
 
 // A row (D/4 vectors) is owned by G = 2^k <= 64 adjacent lanes of ONE wavefront, so the row's
 // lse_acc is read by all of them before one of them rewrites it (program order inside a wave).
@@ -318,11 +288,16 @@ int scratch_for_current_device(void** out) {
 
 }  // namespace
 
-// ---- tile statistics ------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restrict__ pos, const int32_t* __restrict__ seq,
-                                                        int S, int ntiles, int4* __restrict__ out) {
-  const int t = blockIdx.x % ntiles, b = blockIdx.x / ntiles;
-  const int i = t * kAttnTile + threadIdx.x;
+// ---- document masks: the pre-pass ------------------------------------------------------------
+// Three launches per call: (1) the per-64-token statistics of both sides, (2) the visibility bits of the mixed tile
+// pairs and the work counts of the kernels' blocks, (3) the blocks ranked by work.  Each part is a device function over
+// a virtual block index; a launch strings the parts' block ranges together (one wavefront per block).
+
+// (position min, max, sequence id min, max) of tile t of row b
+__device__ __forceinline__ void doc_tile_stats(const int32_t* __restrict__ pos, const int32_t* __restrict__ seq, int S,
+                                               int ntiles, int blk, int lane, int4* __restrict__ out) {
+  const int t = blk % ntiles, b = blk / ntiles;
+  const int i = t * kAttnTile + lane;
   int pmin = 0x7fffffff, pmax = -0x7fffffff - 1, smin = 0x7fffffff, smax = -0x7fffffff - 1;
   if (i < S) {
     const int pp = pos[static_cast<int64_t>(b) * S + i], ss = seq[static_cast<int64_t>(b) * S + i];
@@ -336,9 +311,15 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
     smin = min(smin, __shfl_xor(smin, o, 64));
     smax = max(smax, __shfl_xor(smax, o, 64));
   }
-  if (threadIdx.x == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
+  if (lane == 0) out[static_cast<int64_t>(b) * ntiles + t] = make_int4(pmin, pmax, smin, smax);
 }
 
+__global__ __launch_bounds__(64) void doc_stats_kernel(const AttnParams p, int q_blocks, int4* __restrict__ q_out,
+                                                       int4* __restrict__ k_out) {
+  const int blk = blockIdx.x;
+  if (blk < q_blocks) doc_tile_stats(p.q_pos, p.q_seq, p.Sq, p.nq_stats, blk, threadIdx.x, q_out);
+  else doc_tile_stats(p.k_pos, p.k_seq, p.Sk, p.nk_stats, blk - q_blocks, threadIdx.x, k_out);
+}
 
 // One wavefront per (batch row, 64-query group, kDocBitsChunk key tiles), lane = query of the group.  For each pair of
 // the chunk whose mask the attention kernels evaluate (mixed pairs, and fully visible pairs of a ragged last key tile)
@@ -349,11 +330,10 @@ __global__ __launch_bounds__(64) void tile_stats_kernel(const int32_t* __restric
 constexpr int kDocBitsChunk = 4;
 
 template <bool KEY_MAJOR>
-__global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, int n_chunks, unsigned long long* __restrict__ out,
-                                                      unsigned long long* __restrict__ out_k) {
-  const int chunk = blockIdx.x % n_chunks, bg = blockIdx.x / n_chunks;
+__device__ __forceinline__ void doc_pair_bits(const AttnParams& p, int n_chunks, int blk, int r,
+                                              unsigned long long* __restrict__ out, unsigned long long* __restrict__ out_k) {
+  const int chunk = blk % n_chunks, bg = blk / n_chunks;
   const int g = bg % p.nq_stats, b = bg / p.nq_stats;
-  const int r = threadIdx.x;
   const int4 qs = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + g];
   const int t = chunk * kDocBitsChunk + r;  // lane r < kDocBitsChunk classifies key tile t
   bool mixed = false;
@@ -408,19 +388,33 @@ __global__ __launch_bounds__(64) void doc_bits_kernel(const AttnParams p, int n_
   }
 }
 
-void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st) {
-  if (p.B * p.nq_stats == 0 || p.nk_stats == 0) return;
-  const int n_chunks = (p.nk_stats + kDocBitsChunk - 1) / kDocBitsChunk;
-  const int64_t blocks = static_cast<int64_t>(p.B) * p.nq_stats * n_chunks;
-  MltsKernelTimer timer("attn_doc_bits", st);
-  if (out_k) hipLaunchKernelGGL(doc_bits_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
-  else hipLaunchKernelGGL(doc_bits_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(64), 0, st, p, n_chunks, out, out_k);
+// Number of key tiles that query block qt (`rows` rows: 64, 128 or 256) of batch row b needs (entry qt * B + b): the
+// test of the forward and dQ kernels' scan of the key statistics.
+__device__ __forceinline__ void doc_qblock_work(const AttnParams& p, int rows, int e, int lane, int* __restrict__ work) {
+  const int b = e % p.B, qt = e / p.B;
+  int4 qs[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = qt * (rows >> 6) + i;
+    qs[i] = (i < (rows >> 6) && t < p.nq_stats) ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
+  }
+  int cnt = 0;
+  for (int base = 0; base < p.nk_stats; base += 64) {
+    bool need = false;
+    if (base + lane < p.nk_stats) {
+      const int4 ks = p.k_stats[static_cast<int64_t>(b) * p.nk_stats + base + lane];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) need |= classify_doc_tile(qs[i], ks) != TILE_SKIP;
+    }
+    cnt += __builtin_popcountll(__builtin_amdgcn_ballot_w64(need));
+  }
+  if (lane == 0) work[e] = cnt;
 }
 
-// Number of query tiles that 128-key block kt of batch row b needs (entry kt * B + b): the same test as the dK/dV kernel's
-// scan of the query statistics.  One wavefront per block.
-__global__ __launch_bounds__(64) void doc_kblock_work_kernel(const AttnParams p, int* __restrict__ work) {
-  const int e = blockIdx.x, b = e % p.B, kt = e / p.B, lane = threadIdx.x;
+// Number of query tiles that 128-key block kt of batch row b needs (entry kt * B + b): the test of the dK/dV kernel's
+// scan of the query statistics.
+__device__ __forceinline__ void doc_kblock_work(const AttnParams& p, int e, int lane, int* __restrict__ work) {
+  const int b = e % p.B, kt = e / p.B;
   int4 ks[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -439,10 +433,32 @@ __global__ __launch_bounds__(64) void doc_kblock_work_kernel(const AttnParams p,
   if (lane == 0) work[e] = cnt;
 }
 
+struct DocPairsArgs {
+  int n_chunks, bits_blocks;  // blocks [0, bits_blocks): visibility bits
+  int q_blocks, q_rows;       // then q_blocks query blocks of q_rows rows: work counts into q_work
+  int k_blocks;               // then k_blocks 128-key blocks: work counts into k_work (backward only)
+  unsigned long long *bits, *bits_k;
+  int *q_work, *k_work;
+};
+
+template <bool BACKWARD>
+__global__ __launch_bounds__(64) void doc_pairs_kernel(const AttnParams p, const DocPairsArgs a) {
+  int blk = blockIdx.x;
+  if (blk < a.bits_blocks) {
+    doc_pair_bits<BACKWARD>(p, a.n_chunks, blk, threadIdx.x, a.bits, a.bits_k);
+    return;
+  }
+  blk -= a.bits_blocks;
+  if (blk < a.q_blocks) {
+    doc_qblock_work(p, a.q_rows, blk, threadIdx.x, a.q_work);
+    return;
+  }
+  if (BACKWARD) doc_kblock_work(p, blk - a.q_blocks, threadIdx.x, a.k_work);
+}
+
 // order[rank of i] = i, ranks by work descending (ties by index): every thread counts the entries in front of its own
-__global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ work, int n, int* __restrict__ order) {
-  __shared__ int chunk[256];
-  const int i = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void doc_rank(const int* __restrict__ work, int n, int blk, int* __restrict__ order, int* chunk) {
+  const int i = blk * 256 + threadIdx.x;
   const int wi = i < n ? work[i] : 0;
   int rank = 0;
   for (int base = 0; base < n; base += 256) {
@@ -458,20 +474,76 @@ __global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ 
   if (i < n) order[rank] = i;
 }
 
-void mlts_launch_kblock_order(const AttnParams& p, int* work, int* order, hipStream_t st) {
-  const int n = p.B * ((p.Sk + 127) / 128);
-  if (n == 0) return;
-  MltsKernelTimer timer("attn_doc_order", st);
-  hipLaunchKernelGGL(doc_kblock_work_kernel, dim3(n), dim3(64), 0, st, p, work);
-  hipLaunchKernelGGL(doc_order_kernel, dim3((n + 255) / 256), dim3(256), 0, st, work, n, order);
+// blocks [0, q_grid): the query blocks; then the key blocks (n_k may be 0)
+__global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ q_work, int n_q, int* __restrict__ q_order,
+                                                        int q_grid, const int* __restrict__ k_work, int n_k,
+                                                        int* __restrict__ k_order) {
+  __shared__ int chunk[256];
+  if (static_cast<int>(blockIdx.x) < q_grid) doc_rank(q_work, n_q, blockIdx.x, q_order, chunk);
+  else doc_rank(k_work, n_k, blockIdx.x - q_grid, k_order, chunk);
 }
 
-void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st) {
-  const int ntiles = (S + kAttnTile - 1) / kAttnTile;
-  if (B * ntiles == 0) return;
-  MltsKernelTimer timer("attn_tile_stats", st);
-  hipLaunchKernelGGL(tile_stats_kernel, dim3(B * ntiles), dim3(64), 0, st, pos, seq, S, ntiles, out);
+namespace {
+// Carves the document-mask plan out of the front of the workspace (layout: stats_bytes) and launches the pre-pass.
+char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* ws, hipStream_t st) {
+  if (stats_bytes(s, backward) == 0) return ws;
+  const int64_t B = s->B, nq = p.nq_stats, nk = p.nk_stats;
+  int4* qst = reinterpret_cast<int4*>(ws);
+  ws += align256(B * nq * 16);
+  int4* kst = reinterpret_cast<int4*>(ws);
+  ws += align256(B * nk * 16);
+  DocPairsArgs a{};
+  a.bits = reinterpret_cast<unsigned long long*>(ws);
+  ws += align256(B * nq * nk * 512);
+  if (backward) {
+    a.bits_k = reinterpret_cast<unsigned long long*>(ws);
+    ws += align256(B * nq * nk * 512);
+  }
+  a.q_work = reinterpret_cast<int*>(ws);
+  ws += align256(B * nq * 4);
+  int* q_order = reinterpret_cast<int*>(ws);
+  ws += align256(B * nq * 4);
+  int* k_order = nullptr;
+  if (backward) {
+    a.k_work = reinterpret_cast<int*>(ws);
+    ws += align256(B * ((s->Sk + 127) / 128) * 4);
+    k_order = reinterpret_cast<int*>(ws);
+    ws += align256(B * ((s->Sk + 127) / 128) * 4);
+  }
+  p.q_stats = qst;
+  p.k_stats = kst;
+  p.doc_bits = a.bits;
+  p.doc_bits_k = a.bits_k;
+  if (B * (nq + nk) == 0) return ws;
+  MltsKernelTimer timer("attn_doc_prepass", st);
+  hipLaunchKernelGGL(doc_stats_kernel, dim3(static_cast<unsigned>(B * (nq + nk))), dim3(64), 0, st, p, static_cast<int>(B * nq),
+                     qst, kst);
+  if (B * nq == 0 || nk == 0) return ws;  // no tile pairs
+
+  p.head_pack_shift = mlts_doc_head_pack_shift(s->Hq, s->Hkv);
+  a.q_rows = 256 >> p.head_pack_shift;
+  a.n_chunks = static_cast<int>((nk + kDocBitsChunk - 1) / kDocBitsChunk);
+  a.bits_blocks = static_cast<int>(B * nq * a.n_chunks);
+  a.q_blocks = static_cast<int>(B * ((s->Sq + a.q_rows - 1) / a.q_rows));
+  a.k_blocks = backward ? static_cast<int>(B * ((s->Sk + 127) / 128)) : 0;
+  const bool order_q = a.q_blocks > 1 && a.q_blocks <= kMaxOrderedBlocks;
+  const bool order_k = a.k_blocks > 1 && a.k_blocks <= kMaxOrderedBlocks;
+  if (!order_q) a.q_blocks = 0;
+  if (!order_k) a.k_blocks = 0;
+
+  const unsigned pair_grid = static_cast<unsigned>(a.bits_blocks + a.q_blocks + a.k_blocks);
+  if (backward) hipLaunchKernelGGL(doc_pairs_kernel<true>, dim3(pair_grid), dim3(64), 0, st, p, a);
+  else hipLaunchKernelGGL(doc_pairs_kernel<false>, dim3(pair_grid), dim3(64), 0, st, p, a);
+  if (order_q || order_k) {
+    const int q_grid = (a.q_blocks + 255) / 256, k_grid = (a.k_blocks + 255) / 256;
+    hipLaunchKernelGGL(doc_order_kernel, dim3(q_grid + k_grid), dim3(256), 0, st, a.q_work, a.q_blocks, q_order, q_grid, a.k_work,
+                       a.k_blocks, k_order);
+    if (order_q) p.qblock_order = q_order;
+    if (order_k) p.kblock_order = k_order;
+  }
+  return ws;
 }
+}  // namespace
 
 extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return shape_problem(s); }
 

@@ -105,18 +105,34 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5, l16 = lane & 15;
-  const int nbh = p.B * p.Hq;
+  // Document masks with grouped-query heads: the workgroup's 256 rows are BM >> pack_shift rows of each of
+  // 1 << pack_shift query heads of one KV head (the same rows: the same key tiles), and the (query block, batch row)
+  // pairs are walked in the order of their work, most first (see AttnParams::head_pack_shift, qblock_order).
+  const int pack_shift = MODE == MLTS_MASK_DOC ? p.head_pack_shift : 0;
+  const int rows_per_head = BM >> pack_shift;
+  const int hgroups = p.Hq >> pack_shift;
+  const int nbh = p.B * hgroups;
   const int bid = blockIdx.x;
-  const int qt = p.nqt - 1 - bid / nbh;  // longest (last) q-tiles first under a causal mask
+  int qt = p.nqt - 1 - bid / nbh;  // longest (last) q-tiles first under a causal mask
   const int bh = bid % nbh;
-  const int b = bh / p.Hq, hq = bh % p.Hq;
-  const int hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = qt * BM;
-  const int wq0 = q0 + wave * 32;
+  int b = bh / hgroups;
+  if constexpr (MODE == MLTS_MASK_DOC) {
+    if (p.qblock_order) {
+      const int e = p.qblock_order[(bid / nbh) * p.B + b];
+      qt = e / p.B;
+      b = e % p.B;
+    }
+  }
+  const int hq0 = (bh % hgroups) << pack_shift;  // first head of the workgroup
+  const int hq = MODE == MLTS_MASK_DOC ? hq0 + __builtin_amdgcn_readfirstlane((wave * 32) >> (8 - pack_shift)) : hq0;
+  const int hkv = hq0 / (p.Hq / p.Hkv);
+  const int q0 = qt * rows_per_head;
+  const int wq0 = MODE == MLTS_MASK_DOC ? q0 + ((wave * 32) & (rows_per_head - 1)) : q0 + wave * 32;
   const int qrow = wq0 + l32;
 
-  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
-  const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq * bp.dos[1];
+  // (workgroup tile row -> head hq0 + (row >> (8 - pack_shift)), query q0 + (row & (rows_per_head - 1)))
+  const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq0 * p.qs[1];
+  const bf16_t* dO = static_cast<const bf16_t*>(bp.dout) + b * bp.dos[0] + hq0 * bp.dos[1];
   const bf16_t* K = static_cast<const bf16_t*>(p.k) + b * p.ks[0] + hkv * p.ks[1];
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
 
@@ -139,20 +155,22 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     const int c = tid + n * THREADS;
     const int row = c / CPR;
     const int col = ((c % CPR) ^ swz<D>(row & 15)) * 8;
-    const int64_t r = min(q0 + row, p.Sq - 1);
-    pro_q[n] = *reinterpret_cast<const v4i32*>(Q + r * p.qs[2] + col);
-    pro_d[n] = *reinterpret_cast<const v4i32*>(dO + r * bp.dos[2] + col);
+    const int hrow = MODE == MLTS_MASK_DOC ? row >> (8 - pack_shift) : 0;
+    const int64_t r = min(q0 + (MODE == MLTS_MASK_DOC ? row & (rows_per_head - 1) : row), p.Sq - 1);
+    pro_q[n] = *reinterpret_cast<const v4i32*>(Q + hrow * p.qs[1] + r * p.qs[2] + col);
+    pro_d[n] = *reinterpret_cast<const v4i32*>(dO + hrow * bp.dos[1] + r * bp.dos[2] + col);
   }
   if (fold_stats) {
-    const bf16_t* O = static_cast<const bf16_t*>(p.o) + b * p.os[0] + hq * p.os[1];
+    const bf16_t* O = static_cast<const bf16_t*>(p.o) + b * p.os[0] + hq0 * p.os[1];
     v4i32 pro_o[NPRO];
 #pragma unroll
     for (int n = 0; n < NPRO; ++n) {
       const int c = tid + n * THREADS;
       const int row = c / CPR;
       const int col = ((c % CPR) ^ swz<D>(row & 15)) * 8;
-      const int64_t r = min(q0 + row, p.Sq - 1);
-      pro_o[n] = *reinterpret_cast<const v4i32*>(O + r * p.os[2] + col);
+      const int hrow = MODE == MLTS_MASK_DOC ? row >> (8 - pack_shift) : 0;
+      const int64_t r = min(q0 + (MODE == MLTS_MASK_DOC ? row & (rows_per_head - 1) : row), p.Sq - 1);
+      pro_o[n] = *reinterpret_cast<const v4i32*>(O + hrow * p.os[1] + r * p.os[2] + col);
     }
 #pragma unroll
     for (int n = 0; n < NPRO; ++n) {
@@ -184,7 +202,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #pragma unroll
     for (int w = 0; w < BM / 64; ++w) {
       const int t = (q0 >> 6) + w;
-      bq_stats[w] = t < p.nq_stats ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
+      bq_stats[w] = (w < (rows_per_head >> 6) && t < p.nq_stats) ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t]
+                                                                  : make_int4(0, -1, 0, -1);
     }
     const int t = wq0 >> 6;
     if (t < p.nq_stats) wq_stats = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t];
@@ -561,8 +580,10 @@ int launch(AttnBwdParams bp, hipStream_t st) {
     mlts_set_error("mlts_attn_bwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     return MLTS_ERR_LAUNCH;
   }
-  bp.a.nqt = (bp.a.Sq + BM - 1) / BM;
-  const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * bp.a.Hq;
+  if (MODE != MLTS_MASK_DOC) bp.a.head_pack_shift = 0;  // (set with the block order by the caller's pre-pass otherwise)
+  const int rows = BM >> bp.a.head_pack_shift;
+  bp.a.nqt = (bp.a.Sq + rows - 1) / rows;
+  const int64_t blocks = static_cast<int64_t>(bp.a.nqt) * bp.a.B * (bp.a.Hq >> bp.a.head_pack_shift);
   if (blocks > 0) {
     MltsKernelTimer timer("attn_bwd_dq", st);
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), lds_bytes, st, bp);

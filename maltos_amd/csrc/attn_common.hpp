@@ -40,6 +40,14 @@ struct AttnParams {
   // plain order.
   const int* kblock_order;
   int nqt;              // query tiles per (batch, head) for the launched kernel
+  // Forward with MLTS_MASK_DOC and grouped-query heads: log2 of the number of query heads of one KV head that share a
+  // workgroup (0, 1 or 2).  The workgroup's 256 rows are then 256 >> shift rows of each of those heads: the heads need
+  // the same key tiles, where 256 consecutive rows of one head need the union of the tiles of every document they touch.
+  int head_pack_shift;
+  // Forward with MLTS_MASK_DOC: the (query block of 256 >> head_pack_shift rows, batch row) pairs, index qt * B + b,
+  // sorted by the number of key tiles they need, most first (as kblock_order for the dK/dV kernel).  Null: last blocks
+  // first, the order of a causal mask.
+  const int* qblock_order;
 };
 
 // Backward-only extras.
@@ -142,8 +150,9 @@ __device__ __forceinline__ int doc_scan_class(const DocTileScan& sc, int j) {
   return ((sc.full >> bit) & 1ull) ? TILE_FULL : TILE_MASKED;
 }
 
-void mlts_launch_tile_stats(const int32_t* pos, const int32_t* seq, int B, int S, int4* out, hipStream_t st);
-void mlts_launch_doc_bits(const AttnParams& p, unsigned long long* out, unsigned long long* out_k, hipStream_t st);
-// order[0 .. B * nkt) for AttnParams::kblock_order (nkt = 128-key blocks per row); work: B * nkt ints of scratch
-constexpr int kMaxOrderedBlocks = 8192;
-void mlts_launch_kblock_order(const AttnParams& p, int* work, int* order, hipStream_t st);
+constexpr int kMaxOrderedBlocks = 8192;  // more blocks than this are walked in plain order
+// log2 of the query heads per forward workgroup under a document mask (AttnParams::head_pack_shift)
+inline int mlts_doc_head_pack_shift(int Hq, int Hkv) {
+  const int group = Hq / Hkv;
+  return group % 4 == 0 ? 2 : group % 2 == 0 ? 1 : 0;
+}

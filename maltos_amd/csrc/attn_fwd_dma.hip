@@ -109,14 +109,28 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   // Longest (last) q-tiles first across the whole grid: with causal masks the work per q-tile varies 16:1 and
   // this order keeps the tail short.  (Grouping a head's q-tiles on one XCD for L2 locality was measured: no gain
   // without a mask, 14% slower with the causal mask because of the longer tail.)
-  const int nbh = p.B * p.Hq;
+  // Document masks with grouped-query heads: the workgroup's eight wavefronts are split over 1 << pack_shift query heads
+  // of one KV head, BM >> pack_shift rows of each (the same rows: the same key tiles).
+  const int pack_shift = MODE == MLTS_MASK_DOC ? p.head_pack_shift : 0;
+  const int rows_per_head = BM >> pack_shift;
+  const int hgroups = p.Hq >> pack_shift;
+  const int nbh = p.B * hgroups;
   const int bid = blockIdx.x;
-  const int qt = p.nqt - 1 - bid / nbh;
+  int qt = p.nqt - 1 - bid / nbh;
   const int bh = bid % nbh;
-  const int b = bh / p.Hq, hq = bh % p.Hq;
+  int b = bh / hgroups;
+  if constexpr (MODE == MLTS_MASK_DOC) {
+    // document masks: the (query block, batch row) pairs are walked in the order of their work, most first
+    if (p.qblock_order) {
+      const int e = p.qblock_order[(bid / nbh) * p.B + b];
+      qt = e / p.B;
+      b = e % p.B;
+    }
+  }
+  const int hq = ((bh % hgroups) << pack_shift) + ((wave * 32) >> (8 - pack_shift));
   const int hkv = hq / (p.Hq / p.Hkv);
-  const int q0 = qt * BM;
-  const int wq0 = q0 + wave * 32;
+  const int q0 = qt * rows_per_head;
+  const int wq0 = q0 + ((wave * 32) & (rows_per_head - 1));
   const int qrow = wq0 + l32;
 
   const bf16_t* Q = static_cast<const bf16_t*>(p.q) + b * p.qs[0] + hq * p.qs[1];
@@ -135,7 +149,8 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
 #pragma unroll
     for (int w = 0; w < BM / 64; ++w) {
       const int t = (q0 >> 6) + w;
-      bq_stats[w] = t < p.nq_stats ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t] : make_int4(0, -1, 0, -1);
+      bq_stats[w] = (w < (rows_per_head >> 6) && t < p.nq_stats) ? p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t]
+                                                                  : make_int4(0, -1, 0, -1);
     }
     const int t = wq0 >> 6;
     if (t < p.nq_stats) wq_stats = p.q_stats[static_cast<int64_t>(b) * p.nq_stats + t];
@@ -179,9 +194,9 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       // the visibility words of this wavefront's 32 queries against the tile's keys (256 bytes; read only if the pair is
       // one whose words the pre-pass wrote, i.e. if the wavefront masks the tile)
       if (lane < 16) {
-        const int g = min((q0 >> 6) + (wave >> 1), p.nq_stats - 1);
+        const int g = min(wq0 >> 6, p.nq_stats - 1);
         const unsigned long long* src =
-            p.doc_bits + ((static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats + j) * 64 + (wave & 1) * 32 + lane * 2;
+            p.doc_bits + ((static_cast<int64_t>(b) * p.nq_stats + g) * p.nk_stats + j) * 64 + (wq0 & 32) + lane * 2;
         __builtin_amdgcn_global_load_lds(MLTS_GLB(src), MLTS_LDS(smem + META_OFF + stage * META_BYTES + wave * 256), 16, 0, 0);
       }
     }
@@ -577,8 +592,10 @@ int launch(AttnParams p, hipStream_t st) {
     mlts_set_error("mlts_attn_fwd: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
     return MLTS_ERR_LAUNCH;
   }
-  p.nqt = (p.Sq + BM - 1) / BM;
-  const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * p.Hq;
+  if (MODE != MLTS_MASK_DOC) p.head_pack_shift = 0;  // (set with the block order by the caller's pre-pass otherwise)
+  const int rows = BM >> p.head_pack_shift;
+  p.nqt = (p.Sq + rows - 1) / rows;
+  const int64_t blocks = static_cast<int64_t>(p.nqt) * p.B * (p.Hq >> p.head_pack_shift);
   {
     MltsKernelTimer timer("attn_fwd", st);
     hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(blocks)), dim3(THREADS), lds_bytes, st, p);
