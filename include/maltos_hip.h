@@ -74,6 +74,9 @@ typedef struct mlts_attn_shape {
   const int32_t* k_pos;
   const int32_t* q_seq;
   const int32_t* k_seq;
+  /* MLTS_MASK_DOC only, optional: a plan built by mlts_attn_doc_plan for the same B, Hq, Hkv, Sq, Sk and the same
+   * contents of the four id arrays.  NULL: the call builds its own at the front of its workspace. */
+  const void* doc_plan;
 } mlts_attn_shape;
 
 /* NULL if (dtype, D, mask_mode, strides) is served by a kernel, else a static reason string.
@@ -88,6 +91,18 @@ const char* mlts_attn_supports(const mlts_attn_shape* s);
  * pre-pass forms once per call for all heads: B * Sq * Sk / 8 bytes (forward), twice that (backward). */
 int64_t mlts_attn_fwd_workspace_bytes(const mlts_attn_shape* s);
 int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f32);
+
+/* Document-mask plan: what mlts_attn_fwd and mlts_attn_bwd derive from the ids in front of their kernels (tile
+ * statistics, visibility bits of the tile pairs a document boundary or the diagonal cuts, the order in which the
+ * kernels walk their blocks).  It depends on B, Hq / Hkv, Sq, Sk and the ids only, not on q, k, v: every layer of a
+ * model, forward and backward, attends under the same mask, so a caller can build the plan once per batch into a
+ * buffer of mlts_attn_doc_plan_bytes (16-byte aligned, B * Sq * Sk / 4 bytes and a little) and pass it in
+ * mlts_attn_shape::doc_plan; the calls then skip their pre-pass (three small launches, 28 us at B=2, S=8192) and
+ * mlts_attn_*_workspace_bytes no longer include it.  The plan must not be rewritten while a call that uses it is in
+ * flight.  No counterpart in the reference, whose callers rebuild the varlen metadata per call
+ * (runtime/layers/flash_utils.py:566-640).  Returns 0 bytes / does nothing for shapes the generic kernels serve. */
+int64_t mlts_attn_doc_plan_bytes(const mlts_attn_shape* s);
+int mlts_attn_doc_plan(const mlts_attn_shape* s, void* plan, int64_t plan_bytes, mlts_stream_t stream);
 
 /* Optional trade of memory for matrix work in mlts_attn_bwd: when the caller's workspace is at least
  * mlts_attn_bwd_workspace_bytes + mlts_attn_bwd_ds_handover_bytes, the dK/dV kernel hands dS (bf16, 2 bytes per

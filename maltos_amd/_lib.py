@@ -51,6 +51,7 @@ class AttnShape(C.Structure):
         ("k_pos", C.c_void_p),
         ("q_seq", C.c_void_p),
         ("k_seq", C.c_void_p),
+        ("doc_plan", C.c_void_p),
     ]
 
 
@@ -65,6 +66,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_kernel_timing_enable": (None, [C.c_int]),
     "mlts_kernel_timing_read": (C.c_int, [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     "mlts_attn_supports": (C.c_char_p, [_SHAPE_P]),
+    "mlts_attn_doc_plan_bytes": (C.c_int64, [_SHAPE_P]),
+    "mlts_attn_doc_plan": (C.c_int, [_SHAPE_P, _P, C.c_int64, _P]),
     "mlts_attn_fwd_workspace_bytes": (C.c_int64, [_SHAPE_P]),
     "mlts_attn_bwd_workspace_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
     "mlts_attn_bwd_ds_handover_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),

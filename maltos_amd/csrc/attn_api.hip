@@ -49,8 +49,9 @@ const char* shape_problem(const mlts_attn_shape* s) {
   return nullptr;
 }
 
+// bytes of the document-mask plan at the front of a call's workspace; none when the caller brings the plan
 int64_t stats_bytes(const mlts_attn_shape* s, bool backward) {
-  if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return 0;
+  if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s) || s->doc_plan) return 0;
   const int64_t nq = (s->Sq + kAttnTile - 1) / kAttnTile, nk = (s->Sk + kAttnTile - 1) / kAttnTile;
   // tile statistics of both sides, then the visibility bits of the mixed (query group, key tile) pairs (512 bytes per
   // pair, indexed densely: Sq * Sk / 8 bytes per batch row), query-major and, for the backward pass, key-major as well
@@ -484,9 +485,16 @@ __global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ 
 }
 
 namespace {
-// Carves the document-mask plan out of the front of the workspace (layout: stats_bytes) and launches the pre-pass.
+// The document-mask plan at the front of a call's workspace (layout: stats_bytes), or the one the caller brought
+// (s->doc_plan, always in the backward's layout): sets the plan pointers of p; builds the plan unless it was brought.
 char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* ws, hipStream_t st) {
-  if (stats_bytes(s, backward) == 0) return ws;
+  if (s->mask_mode != MLTS_MASK_DOC || !uses_mfma(s)) return ws;
+  const bool brought = s->doc_plan != nullptr;
+  char* const ws_in = ws;
+  if (brought) {
+    ws = static_cast<char*>(const_cast<void*>(s->doc_plan));
+    backward = true;
+  }
   const int64_t B = s->B, nq = p.nq_stats, nk = p.nk_stats;
   int4* qst = reinterpret_cast<int4*>(ws);
   ws += align256(B * nq * 16);
@@ -510,27 +518,30 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* 
     k_order = reinterpret_cast<int*>(ws);
     ws += align256(B * ((s->Sk + 127) / 128) * 4);
   }
+  char* const ws_out = brought ? ws_in : ws;
   p.q_stats = qst;
   p.k_stats = kst;
   p.doc_bits = a.bits;
   p.doc_bits_k = a.bits_k;
-  if (B * (nq + nk) == 0) return ws;
-  MltsKernelTimer timer("attn_doc_prepass", st);
-  hipLaunchKernelGGL(doc_stats_kernel, dim3(static_cast<unsigned>(B * (nq + nk))), dim3(64), 0, st, p, static_cast<int>(B * nq),
-                     qst, kst);
-  if (B * nq == 0 || nk == 0) return ws;  // no tile pairs
-
   p.head_pack_shift = mlts_doc_head_pack_shift(s->Hq, s->Hkv);
   a.q_rows = 256 >> p.head_pack_shift;
   a.n_chunks = static_cast<int>((nk + kDocBitsChunk - 1) / kDocBitsChunk);
   a.bits_blocks = static_cast<int>(B * nq * a.n_chunks);
   a.q_blocks = static_cast<int>(B * ((s->Sq + a.q_rows - 1) / a.q_rows));
   a.k_blocks = backward ? static_cast<int>(B * ((s->Sk + 127) / 128)) : 0;
-  const bool order_q = a.q_blocks > 1 && a.q_blocks <= kMaxOrderedBlocks;
-  const bool order_k = a.k_blocks > 1 && a.k_blocks <= kMaxOrderedBlocks;
+  const bool pairs = B * nq > 0 && nk > 0;
+  const bool order_q = pairs && a.q_blocks > 1 && a.q_blocks <= kMaxOrderedBlocks;
+  const bool order_k = pairs && a.k_blocks > 1 && a.k_blocks <= kMaxOrderedBlocks;
   if (!order_q) a.q_blocks = 0;
   if (!order_k) a.k_blocks = 0;
+  if (order_q) p.qblock_order = q_order;
+  if (order_k) p.kblock_order = k_order;
+  if (brought || B * (nq + nk) == 0) return ws_out;
 
+  MltsKernelTimer timer("attn_doc_prepass", st);
+  hipLaunchKernelGGL(doc_stats_kernel, dim3(static_cast<unsigned>(B * (nq + nk))), dim3(64), 0, st, p, static_cast<int>(B * nq),
+                     qst, kst);
+  if (!pairs) return ws_out;
   const unsigned pair_grid = static_cast<unsigned>(a.bits_blocks + a.q_blocks + a.k_blocks);
   if (backward) hipLaunchKernelGGL(doc_pairs_kernel<true>, dim3(pair_grid), dim3(64), 0, st, p, a);
   else hipLaunchKernelGGL(doc_pairs_kernel<false>, dim3(pair_grid), dim3(64), 0, st, p, a);
@@ -538,12 +549,34 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* 
     const int q_grid = (a.q_blocks + 255) / 256, k_grid = (a.k_blocks + 255) / 256;
     hipLaunchKernelGGL(doc_order_kernel, dim3(q_grid + k_grid), dim3(256), 0, st, a.q_work, a.q_blocks, q_order, q_grid, a.k_work,
                        a.k_blocks, k_order);
-    if (order_q) p.qblock_order = q_order;
-    if (order_k) p.kblock_order = k_order;
   }
-  return ws;
+  return ws_out;
 }
 }  // namespace
+
+extern "C" int64_t mlts_attn_doc_plan_bytes(const mlts_attn_shape* s) {
+  if (shape_problem(s)) return -1;
+  mlts_attn_shape t = *s;
+  t.doc_plan = nullptr;
+  return stats_bytes(&t, true);
+}
+
+extern "C" int mlts_attn_doc_plan(const mlts_attn_shape* s, void* plan, int64_t plan_bytes, mlts_stream_t stream) {
+  const char* why = shape_problem(s);
+  MLTS_REQUIRE(why == nullptr, "mlts_attn_doc_plan: %s", why);
+  MLTS_REQUIRE(s->mask_mode == MLTS_MASK_DOC, "mlts_attn_doc_plan: mask_mode must be MLTS_MASK_DOC");
+  mlts_attn_shape t = *s;
+  t.doc_plan = nullptr;
+  const int64_t need = stats_bytes(&t, true);
+  if (need == 0) return MLTS_OK;  // a shape the generic kernels serve: they evaluate the mask themselves
+  MLTS_REQUIRE(plan && plan_bytes >= need, "mlts_attn_doc_plan: plan buffer too small (%lld < %lld)", (long long)plan_bytes,
+               (long long)need);
+  MLTS_REQUIRE(mlts_aligned16(plan), "mlts_attn_doc_plan: the plan buffer must be 16-byte aligned");
+  AttnParams p;
+  fill_params(p, &t, nullptr, nullptr, nullptr, nullptr, nullptr);
+  setup_stats(p, &t, true, static_cast<char*>(plan), static_cast<hipStream_t>(stream));
+  return mlts_check_launch("mlts_attn_doc_plan");
+}
 
 extern "C" const char* mlts_attn_supports(const mlts_attn_shape* s) { return shape_problem(s); }
 

@@ -99,6 +99,54 @@ def _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq) -> Att
     return s
 
 
+# Document-mask plans (mlts_attn_doc_plan): every layer of a model, forward and backward, attends under the same ids, so
+# the plan of a call is kept and handed to later calls with the same ids.  "The same" is judged without reading
+# device memory: same address, dtype, shape, strides and autograd version of the four id tensors as given by the caller,
+# which are kept alive with the plan so that their addresses cannot be handed to other tensors meanwhile (an in-place
+# change of the ids through torch bumps the version; writes behind torch's back are not seen: clear_doc_plan_cache()).
+_DOC_PLAN_CACHE: list[tuple[tuple, tuple, torch.Tensor]] = []
+_DOC_PLAN_CACHE_ENTRIES = 8
+
+
+def set_doc_plan_cache_entries(n: int) -> int:
+    """Number of document-mask plans kept (0: every call builds its own in its workspace).  Returns the previous value."""
+    global _DOC_PLAN_CACHE_ENTRIES
+    if n < 0:
+        raise ValueError("the number of cached plans is >= 0")
+    previous, _DOC_PLAN_CACHE_ENTRIES = _DOC_PLAN_CACHE_ENTRIES, int(n)
+    del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
+    return previous
+
+
+def clear_doc_plan_cache() -> None:
+    _DOC_PLAN_CACHE.clear()
+
+
+def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.device) -> torch.Tensor | None:
+    """Sets shape.doc_plan to a kept plan for these ids, building it first if there is none.  `given`: the caller's id
+    tensors, `used`: their int32 forms that shape points at.  Returns the plan (to be kept alive over the launch)."""
+    if shape.mask_mode != MASK_DOC or _DOC_PLAN_CACHE_ENTRIES == 0 or torch.cuda.is_current_stream_capturing():
+        return None  # (a captured graph must rebuild the plan on every replay: its id buffers are refilled in place)
+    L = _lib.lib()
+    nbytes = L.mlts_attn_doc_plan_bytes(C.byref(shape))
+    if nbytes <= 0:
+        return None
+    key = (shape.B, shape.Hq, shape.Hkv, shape.Sq, shape.Sk, shape.D, shape.dtype, device, torch.cuda.current_stream().cuda_stream,
+           tuple((t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride())) for t in given))
+    for i, (k_, _, plan) in enumerate(_DOC_PLAN_CACHE):
+        if k_ == key:
+            if i:
+                _DOC_PLAN_CACHE.insert(0, _DOC_PLAN_CACHE.pop(i))
+            shape.doc_plan = plan.data_ptr()
+            return plan
+    plan = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+    _lib.check(L.mlts_attn_doc_plan(C.byref(shape), _p(plan), nbytes, _stream()))
+    _DOC_PLAN_CACHE.insert(0, (key, tuple(given) + tuple(used), plan))
+    del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
+    shape.doc_plan = plan.data_ptr()
+    return plan
+
+
 def _bshd_empty(B: int, H: int, S: int, D: int, like: torch.Tensor, dtype=None) -> torch.Tensor:
     """[B, H, S, D] view over [B, S, H, D] storage: the layout LlamaAttention transposes back to."""
     return torch.empty((B, S, H, D), dtype=dtype or like.dtype, device=like.device).transpose(1, 2)
@@ -119,6 +167,7 @@ def attention_forward(q, k, v, *, mask_mode: int, scale: float | None = None, q_
     lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
     if B == 0 or Sq == 0:
         return o, lse
+    given = (q_pos, k_pos, q_seq, k_seq)
     q_pos, q_seq = _ids32(q_pos, B, Sq, "q_positions"), _ids32(q_seq, B, Sq, "q_sequence_ids")
     k_pos, k_seq = _ids32(k_pos, B, k.size(2), "k_positions"), _ids32(k_seq, B, k.size(2), "k_sequence_ids")
     shape = _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
@@ -126,6 +175,7 @@ def attention_forward(q, k, v, *, mask_mode: int, scale: float | None = None, q_
     why = L.mlts_attn_supports(C.byref(shape))
     if why:
         raise ValueError(f"attention_forward: {why.decode()}")
+    plan = _attach_doc_plan(shape, given, (q_pos, k_pos, q_seq, k_seq), q.device)  # noqa: F841 (alive over the launch)
     ws_bytes = L.mlts_attn_fwd_workspace_bytes(C.byref(shape))
     ws = _workspace(ws_bytes, q.device)
     _lib.check(L.mlts_attn_fwd(C.byref(shape), _p(q), _p(k), _p(v), _p(o), _p(lse), _p(ws), ws_bytes, _stream()))
@@ -164,6 +214,7 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
         raise ValueError(f"softmax_lse must be float32 of shape {(B, Hq, Sq)}, got {lse.dtype} {tuple(lse.shape)}")
     lse = lse.contiguous()
     scale = D ** -0.5 if scale is None else scale
+    given = (q_pos, k_pos, q_seq, k_seq)
     q_pos, q_seq = _ids32(q_pos, B, Sq, "q_positions"), _ids32(q_seq, B, Sq, "q_sequence_ids")
     k_pos, k_seq = _ids32(k_pos, B, Sk, "k_positions"), _ids32(k_seq, B, Sk, "k_sequence_ids")
     shape = _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
@@ -171,6 +222,7 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
     why = L.mlts_attn_supports(C.byref(shape))
     if why:
         raise ValueError(f"attention_backward: {why.decode()}")
+    plan = _attach_doc_plan(shape, given, (q_pos, k_pos, q_seq, k_seq), q.device)  # noqa: F841 (alive over the launch)
     ws_bytes = L.mlts_attn_bwd_workspace_bytes(C.byref(shape), int(accumulate))
     if _BWD_DS_HANDOVER_MAX_BYTES > 0:
         ds_bytes = L.mlts_attn_bwd_ds_handover_bytes(C.byref(shape), int(accumulate))

@@ -125,6 +125,46 @@ def test_document_mask_many_tiles(dev, D):
     run_case(dev, torch.bfloat16, 1, 1, 1, S, S, D, ops.MASK_DOC, 32 + D, ids=(pos.view(1, S), seq.view(1, S)), share_ids=False)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_document_plan_is_reused_and_follows_the_ids(dev, D):
+    """The plan built for a call's ids (mlts_attn_doc_plan) serves later calls with the same id tensors, gives the results
+    of a call that builds its own, bit for bit, and is not used once the ids have changed in place."""
+    B, Hq, Hkv, S = 2, 4, 1, 330
+    gen = torch.Generator().manual_seed(90 + D)
+    q, k, v, do = bshd(B, Hq, S, D, gen, torch.bfloat16), bshd(B, Hkv, S, D, gen, torch.bfloat16), \
+        bshd(B, Hkv, S, D, gen, torch.bfloat16), bshd(B, Hq, S, D, gen, torch.bfloat16)
+    pos, seq = make_docs(B, S, gen, 90, pad_tail=5)
+    dpos, dseq = pos.int().to(dev), seq.int().to(dev)
+
+    def run():
+        qg, kg, vg = (t.detach().to(dev).requires_grad_(True) for t in (q, k, v))
+        o = ops.attention(qg, kg, vg, mask_mode=ops.MASK_DOC, q_pos=dpos, k_pos=dpos, q_seq=dseq, k_seq=dseq)
+        o.backward(do.to(dev))
+        return o.detach(), qg.grad, kg.grad, vg.grad
+
+    ops.clear_doc_plan_cache()
+    first = run()
+    assert len(ops._DOC_PLAN_CACHE) == 1
+    again = run()
+    assert len(ops._DOC_PLAN_CACHE) == 1
+    previous = ops.set_doc_plan_cache_entries(0)
+    try:
+        own = run()  # forward and backward each build the plan in their workspace
+    finally:
+        ops.set_doc_plan_cache_entries(previous)
+    for a, b_, c in zip(first, again, own):
+        assert torch.equal(a, b_) and torch.equal(a, c)
+    run()  # (disabling dropped the entry: keep one again, for the old ids)
+    assert len(ops._DOC_PLAN_CACHE) == 1
+    pos2, seq2 = make_docs(B, S, gen, 40, pad_tail=17)
+    dpos.copy_(pos2)
+    dseq.copy_(seq2)
+    o2 = run()[0]
+    assert len(ops._DOC_PLAN_CACHE) == 2  # same tensors, another version: a new plan beside the old one
+    want, _ = oa.attention_with_lse(q.float(), k.float(), v.float(), oa.doc_mask(pos2, pos2, seq2, seq2))
+    check(o2, want, torch.bfloat16, "O after the ids changed in place")
+
+
 @pytest.mark.parametrize("D", [1, 3, 24, 96, 192])
 def test_generic_head_dims(dev, D):
     run_case(dev, torch.float32, 1, 2, 1, 70, 70, D, ops.MASK_CAUSAL, seed=D)

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(str(_lib.LIB_PATH))
     for name in names:
         assert hasattr(handle, name), f"{name} not exported by {_lib.LIB_PATH.name}"
-    assert _lib.lib().mlts_abi_version() == 2
+    assert _lib.lib().mlts_abi_version() == 3
 
 
 def test_entry_points_validate_before_launch():
