@@ -547,6 +547,23 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ swz<D>(row & 15)) << 4));
       if (wq0 + row < p.Sq) *reinterpret_cast<v4i32*>(obase + static_cast<int64_t>(wq0 + row) * bp.dqs[2] + chunk * 8) = x;
     }
+  } else if (qrow < p.Sq && bp.accumulate_f32) {
+    // fp32 gradients that are added to (ring steps): all loads of the old values before the first store, one memory
+    // round trip instead of sixteen dependent ones
+    f32x4* dst = reinterpret_cast<f32x4*>(bp.dq_acc + b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(qrow) * bp.dqs[2] + hh * 4);
+    f32x4 cur[DB][4];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) cur[db][g] = dst[db * 8 + g * 2];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cur[db][g][r] += dqacc[db][g * 4 + r] * oscale;
+        dst[db * 8 + g * 2] = cur[db][g];
+      }
   } else if (qrow < p.Sq) {
     const int64_t rowoff = b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(qrow) * bp.dqs[2];
 #pragma unroll
@@ -554,18 +571,10 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = db * 32 + g * 8 + hh * 4;
-        if (bp.accumulate_f32) {
-          f32x4* dst = reinterpret_cast<f32x4*>(bp.dq_acc + rowoff + d);
-          f32x4 cur = *dst;
+        bf16x4 w;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) cur[r] += dqacc[db][g * 4 + r] * oscale;
-          *dst = cur;
-        } else {
-          bf16x4 w;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(dqacc[db][g * 4 + r] * oscale);
-          *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(bp.dq_acc) + rowoff + d) = w;
-        }
+        for (int r = 0; r < 4; ++r) w[r] = static_cast<bf16_t>(dqacc[db][g * 4 + r] * oscale);
+        *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(bp.dq_acc) + rowoff + d) = w;
       }
     }
   }

@@ -756,6 +756,26 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ (((row >> 2) & 1) << 2)) << 4));
         if (wkv0 + row < p.Sk) *reinterpret_cast<v4i32*>(obase + static_cast<int64_t>(wkv0 + row) * os[2] + chunk * 8) = x;
       }
+    } else if (bp.accumulate_f32) {
+      // fp32 gradients that are added to (ring steps): every load of the old values is issued before the first store,
+      // so that the 64 read-modify-writes of a lane are one memory round trip and not 64 dependent ones (a store
+      // between two loads through the same pointer keeps the compiler from moving the second load up)
+      float* obase = static_cast<float*>(optr) + b * os[0] + hkv * os[1] + l32;
+      float cur[DB][16];
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
+          cur[db][e] = row < p.Sk ? obase[static_cast<int64_t>(row) * os[2] + db * 32] : 0.f;
+        }
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
+          if (row < p.Sk) obase[static_cast<int64_t>(row) * os[2] + db * 32] = cur[db][e] + acc[db][e] * oscale;
+        }
     } else {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
@@ -765,8 +785,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
           const int row = wkv0 + (e >> 2) * 8 + hh * 4 + (e & 3);
           if (row < p.Sk) {
             const int64_t o = b * os[0] + hkv * os[1] + static_cast<int64_t>(row) * os[2] + d;
-            if (bp.accumulate_f32) static_cast<float*>(optr)[o] += acc[db][e] * oscale;
-            else static_cast<bf16_t*>(optr)[o] = static_cast<bf16_t>(acc[db][e] * oscale);
+            static_cast<bf16_t*>(optr)[o] = static_cast<bf16_t>(acc[db][e] * oscale);
           }
         }
       }
