@@ -46,6 +46,18 @@ def zigzag_ring_schedule(rank: int, world_size: int) -> list[tuple[int, str]]:
     return plan
 
 
+def _chunk_grad_buffers(ks, device):
+    """Zeroed fp32 dK, dV of every chunk: [2 * chunks, ...] in one buffer when the chunks have one shape (one fill and
+    one conversion instead of two per chunk), else a list."""
+    if all(k.shape == ks[0].shape for k in ks):
+        return torch.zeros((2 * len(ks), *ks[0].shape), dtype=torch.float32, device=device)
+    return [torch.zeros(k.shape, dtype=torch.float32, device=device) for k in ks for _ in range(2)]
+
+
+def _chunk_grads(dkv, dtype):
+    return dkv.to(dtype).unbind(0) if isinstance(dkv, torch.Tensor) else [g.to(dtype) for g in dkv]
+
+
 class _ZigzagRingFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q: torch.Tensor, rank: int, world_size: int, *kv_flat: torch.Tensor):
@@ -81,11 +93,10 @@ class _ZigzagRingFunction(torch.autograd.Function):
         half = q.size(-2) // 2
         dout = dout.contiguous()
         dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-        grads: list[torch.Tensor | None] = [None] * (2 * world_size)
+        dkv = _chunk_grad_buffers(kv_flat[0::2], q.device)
         for src, kind in zigzag_ring_schedule(rank, world_size):
             k, v = kv_flat[2 * src], kv_flat[2 * src + 1]
-            dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
-            dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+            dk, dv = dkv[2 * src], dkv[2 * src + 1]
             if kind == "causal":
                 ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dk, dv, mask_mode=ops.MASK_CAUSAL)
             elif kind == "front_kv":
@@ -95,9 +106,7 @@ class _ZigzagRingFunction(torch.autograd.Function):
                 ops.attention_backward_accumulate(dout[:, :, half:], q[:, :, half:], k, v, out[:, :, half:],
                                                   lse[:, :, half:].contiguous(), dq[:, :, half:], dk, dv,
                                                   mask_mode=ops.MASK_NONE)
-            grads[2 * src] = dk.to(k.dtype)
-            grads[2 * src + 1] = dv.to(v.dtype)
-        return (dq.to(q.dtype), None, None, *grads)
+        return (dq.to(q.dtype), None, None, *_chunk_grads(dkv, kv_flat[0].dtype))
 
 
 class _PackedRingFunction(torch.autograd.Function):
@@ -127,15 +136,15 @@ class _PackedRingFunction(torch.autograd.Function):
         dout = dout.contiguous()
         dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
         grads: list[torch.Tensor | None] = [None] * (4 * world_size)
+        dkv = _chunk_grad_buffers(flat[0::4], q.device)
         for step in range(world_size):
             src = (rank - step) % world_size
             k, v, k_pos, k_seq = flat[4 * src:][:4]
-            dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
-            dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
-            ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dk, dv, mask_mode=ops.MASK_DOC, q_pos=q_pos,
-                                              k_pos=k_pos, q_seq=q_seq, k_seq=k_seq)
-            grads[4 * src] = dk.to(k.dtype)
-            grads[4 * src + 1] = dv.to(v.dtype)
+            ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dkv[2 * src], dkv[2 * src + 1], mask_mode=ops.MASK_DOC,
+                                              q_pos=q_pos, k_pos=k_pos, q_seq=q_seq, k_seq=k_seq)
+        dkv = _chunk_grads(dkv, flat[0].dtype)
+        for src in range(world_size):
+            grads[4 * src], grads[4 * src + 1] = dkv[2 * src], dkv[2 * src + 1]
         return (dq.to(q.dtype), None, None, None, None, *grads)
 
 
