@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import threading
 
 import torch
 
@@ -106,6 +107,7 @@ def _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq) -> Att
 # change of the ids through torch bumps the version; writes behind torch's back are not seen: clear_doc_plan_cache()).
 _DOC_PLAN_CACHE: list[tuple[tuple, tuple, torch.Tensor]] = []
 _DOC_PLAN_CACHE_ENTRIES = 8
+_DOC_PLAN_LOCK = threading.Lock()  # forward runs on the caller's thread, backward on autograd's device thread
 
 
 def set_doc_plan_cache_entries(n: int) -> int:
@@ -113,13 +115,15 @@ def set_doc_plan_cache_entries(n: int) -> int:
     global _DOC_PLAN_CACHE_ENTRIES
     if n < 0:
         raise ValueError("the number of cached plans is >= 0")
-    previous, _DOC_PLAN_CACHE_ENTRIES = _DOC_PLAN_CACHE_ENTRIES, int(n)
-    del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
+    with _DOC_PLAN_LOCK:
+        previous, _DOC_PLAN_CACHE_ENTRIES = _DOC_PLAN_CACHE_ENTRIES, int(n)
+        del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
     return previous
 
 
 def clear_doc_plan_cache() -> None:
-    _DOC_PLAN_CACHE.clear()
+    with _DOC_PLAN_LOCK:
+        _DOC_PLAN_CACHE.clear()
 
 
 def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.device) -> torch.Tensor | None:
@@ -133,18 +137,19 @@ def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.
         return None
     key = (shape.B, shape.Hq, shape.Hkv, shape.Sq, shape.Sk, shape.D, shape.dtype, device, torch.cuda.current_stream().cuda_stream,
            tuple((t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride())) for t in given))
-    for i, (k_, _, plan) in enumerate(_DOC_PLAN_CACHE):
-        if k_ == key:
-            if i:
-                _DOC_PLAN_CACHE.insert(0, _DOC_PLAN_CACHE.pop(i))
-            shape.doc_plan = plan.data_ptr()
-            return plan
-    plan = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-    _lib.check(L.mlts_attn_doc_plan(C.byref(shape), _p(plan), nbytes, _stream()))
-    _DOC_PLAN_CACHE.insert(0, (key, tuple(given) + tuple(used), plan))
-    del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
-    shape.doc_plan = plan.data_ptr()
-    return plan
+    with _DOC_PLAN_LOCK:
+        for i, (k_, _, plan) in enumerate(_DOC_PLAN_CACHE):
+            if k_ == key:
+                if i:
+                    _DOC_PLAN_CACHE.insert(0, _DOC_PLAN_CACHE.pop(i))
+                shape.doc_plan = plan.data_ptr()
+                return plan
+        plan = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _lib.check(L.mlts_attn_doc_plan(C.byref(shape), _p(plan), nbytes, _stream()))
+        _DOC_PLAN_CACHE.insert(0, (key, tuple(given) + tuple(used), plan))
+        del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
+        shape.doc_plan = plan.data_ptr()
+        return plan
 
 
 def _bshd_empty(B: int, H: int, S: int, D: int, like: torch.Tensor, dtype=None) -> torch.Tensor:
