@@ -125,6 +125,19 @@ def test_document_mask_many_tiles(dev, D):
     run_case(dev, torch.bfloat16, 1, 1, 1, S, S, D, ops.MASK_DOC, 32 + D, ids=(pos.view(1, S), seq.view(1, S)), share_ids=False)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_document_mask_drawn_shapes(dev, seed):
+    """Drawn batch sizes, head groupings (1, 2, 3, 4, 8 query heads per KV head: the forward and dQ workgroups take one,
+    two or four heads), ragged lengths and document lengths, both head dims, ids shared between the sides or not."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+    draw = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    B, Hkv, group = draw(1, 3), draw(1, 2), (1, 2, 3, 4, 8)[draw(0, 4)]
+    S = (draw(1, 63), draw(64, 300), draw(301, 900))[draw(0, 2)]
+    D = (64, 128)[seed % 2]
+    run_case(dev, torch.bfloat16, B, Hkv * group, Hkv, S, S, D, ops.MASK_DOC, 2000 + seed, max_doc=draw(1, max(1, S // 2)),
+             pad_tail=draw(0, min(40, S - 1)), share_ids=bool(seed % 3))
+
+
 @pytest.mark.parametrize("D", [64, 128])
 def test_document_plan_is_reused_and_follows_the_ids(dev, D):
     """The plan built for a call's ids (mlts_attn_doc_plan) serves later calls with the same id tensors, gives the results
