@@ -466,10 +466,16 @@ __device__ __forceinline__ void doc_rank(const int* __restrict__ work, int n, in
     __syncthreads();
     chunk[threadIdx.x] = base + threadIdx.x < n ? work[base + threadIdx.x] : -1;
     __syncthreads();
-    const int m = min(256, n - base);
-    for (int j = 0; j < m; ++j) {
-      const int wj = chunk[j];
-      rank += (wj > wi || (wj == wi && base + j < i)) ? 1 : 0;
+    // (entries past n hold -1: never in front of an entry, whose count is >= 0)
+    const int4* chunk4 = reinterpret_cast<const int4*>(chunk);
+#pragma unroll 4
+    for (int j = 0; j < 64; ++j) {
+      const int4 w = chunk4[j];
+      const int at = base + 4 * j;
+      rank += (w.x > wi || (w.x == wi && at < i)) ? 1 : 0;
+      rank += (w.y > wi || (w.y == wi && at + 1 < i)) ? 1 : 0;
+      rank += (w.z > wi || (w.z == wi && at + 2 < i)) ? 1 : 0;
+      rank += (w.w > wi || (w.w == wi && at + 3 < i)) ? 1 : 0;
     }
   }
   if (i < n) order[rank] = i;
@@ -479,7 +485,7 @@ __device__ __forceinline__ void doc_rank(const int* __restrict__ work, int n, in
 __global__ __launch_bounds__(256) void doc_order_kernel(const int* __restrict__ q_work, int n_q, int* __restrict__ q_order,
                                                         int q_grid, const int* __restrict__ k_work, int n_k,
                                                         int* __restrict__ k_order) {
-  __shared__ int chunk[256];
+  __shared__ __attribute__((aligned(16))) int chunk[256];
   if (static_cast<int>(blockIdx.x) < q_grid) doc_rank(q_work, n_q, blockIdx.x, q_order, chunk);
   else doc_rank(k_work, n_k, blockIdx.x - q_grid, k_order, chunk);
 }
