@@ -107,6 +107,7 @@ def _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq) -> Att
 # change of the ids through torch bumps the version; writes behind torch's back are not seen: clear_doc_plan_cache()).
 _DOC_PLAN_CACHE: list[tuple[tuple, tuple, torch.Tensor]] = []
 _DOC_PLAN_CACHE_ENTRIES = 8
+_DOC_PLAN_CACHE_BYTES = 1 << 30  # most bytes of plans kept (a plan is B * Sq * Sk / 4 bytes); larger plans are not kept
 _DOC_PLAN_LOCK = threading.Lock()  # forward runs on the caller's thread, backward on autograd's device thread
 
 
@@ -133,7 +134,7 @@ def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.
         return None  # (a captured graph must rebuild the plan on every replay: its id buffers are refilled in place)
     L = _lib.lib()
     nbytes = L.mlts_attn_doc_plan_bytes(C.byref(shape))
-    if nbytes <= 0:
+    if nbytes <= 0 or nbytes > _DOC_PLAN_CACHE_BYTES:
         return None
     key = (shape.B, shape.Hq, shape.Hkv, shape.Sq, shape.Sk, shape.D, shape.dtype, device, torch.cuda.current_stream().cuda_stream,
            tuple((t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride())) for t in given))
@@ -148,6 +149,8 @@ def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.
         _lib.check(L.mlts_attn_doc_plan(C.byref(shape), _p(plan), nbytes, _stream()))
         _DOC_PLAN_CACHE.insert(0, (key, tuple(given) + tuple(used), plan))
         del _DOC_PLAN_CACHE[_DOC_PLAN_CACHE_ENTRIES:]
+        while sum(e[2].numel() for e in _DOC_PLAN_CACHE) > _DOC_PLAN_CACHE_BYTES:
+            _DOC_PLAN_CACHE.pop()
         shape.doc_plan = plan.data_ptr()
         return plan
 
