@@ -136,6 +136,8 @@ def _attach_doc_plan(shape: AttnShape, given: tuple, used: tuple, device: torch.
     nbytes = L.mlts_attn_doc_plan_bytes(C.byref(shape))
     if nbytes <= 0 or nbytes > _DOC_PLAN_CACHE_BYTES:
         return None
+    if any(t.is_inference() for t in given):
+        return None  # (inference tensors carry no version counter: nothing tells a rewritten id tensor from the old one)
     key = (shape.B, shape.Hq, shape.Hkv, shape.Sq, shape.Sk, shape.D, shape.dtype, device, torch.cuda.current_stream().cuda_stream,
            tuple((t.data_ptr(), t._version, t.dtype, tuple(t.shape), tuple(t.stride())) for t in given))
     with _DOC_PLAN_LOCK:
