@@ -169,6 +169,11 @@ def test_document_plan_is_reused_and_follows_the_ids(dev, D):
         assert torch.equal(a, b_) and torch.equal(a, c)
     run()  # (disabling dropped the entry: keep one again, for the old ids)
     assert len(ops._DOC_PLAN_CACHE) == 1
+    with torch.inference_mode():  # id tensors without a version counter: served, never kept
+        ipos, iseq = pos.int().to(dev), seq.int().to(dev)
+        o_inf = ops.attention(q.to(dev), k.to(dev), v.to(dev), mask_mode=ops.MASK_DOC, q_pos=ipos, k_pos=ipos, q_seq=iseq,
+                              k_seq=iseq)
+    assert torch.equal(o_inf, first[0]) and len(ops._DOC_PLAN_CACHE) == 1
     pos2, seq2 = make_docs(B, S, gen, 40, pad_tail=17)
     dpos.copy_(pos2)
     dseq.copy_(seq2)
