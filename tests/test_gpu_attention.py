@@ -125,6 +125,30 @@ def test_document_mask_many_tiles(dev, D):
     run_case(dev, torch.bfloat16, 1, 1, 1, S, S, D, ops.MASK_DOC, 32 + D, ids=(pos.view(1, S), seq.view(1, S)), share_ids=False)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_document_mask_long_row_equals_causal_attention_per_document(dev, D):
+    """A size the oracle does not reach (32768 tokens): packed documents attend exactly as each document alone under the
+    causal mask, forward and backward, so the document kernels are checked against the causal kernels slice by slice."""
+    S, Hq, Hkv = 32768, 4, 2
+    gen = torch.Generator().manual_seed(7 + D)
+    q, k, v, do = (bshd(1, h, S, D, gen, torch.bfloat16).to(dev) for h in (Hq, Hkv, Hkv, Hq))
+    cuts = [0, 1, 4097, 4160, 12352, 12353, 20000, 28671, S]  # one-token documents, cuts on and off tile edges
+    pos = torch.cat([torch.arange(b - a) for a, b in zip(cuts, cuts[1:])]).view(1, S).int().to(dev)
+    seq = torch.cat([torch.full((b - a,), i) for i, (a, b) in enumerate(zip(cuts, cuts[1:]))]).view(1, S).int().to(dev)
+    ids = dict(q_pos=pos, k_pos=pos, q_seq=seq, k_seq=seq)
+    o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, **ids)
+    dq, dk, dv = ops.attention_backward(do, q, k, v, o, lse, mask_mode=ops.MASK_DOC, **ids)
+    for a, b in zip(cuts, cuts[1:]):
+        sl = (slice(None), slice(None), slice(a, b))
+        o1, lse1 = ops.attention_forward(q[sl], k[sl], v[sl], mask_mode=ops.MASK_CAUSAL)
+        g1 = ops.attention_backward(do[sl], q[sl], k[sl], v[sl], o1, lse1, mask_mode=ops.MASK_CAUSAL)
+        tag = f"D{D} document [{a}, {b})"
+        check(o[sl], o1, torch.bfloat16, tag + " O")
+        assert (lse[:, :, a:b] - lse1).abs().max() <= 4e-3, tag + " LSE (two kernel results, each within 2e-3)"
+        for got, want, name in zip((dq, dk, dv), g1, ("dQ", "dK", "dV")):
+            check(got[sl], want, torch.bfloat16, f"{tag} {name}")
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_document_mask_drawn_shapes(dev, seed):
     """Drawn batch sizes, head groupings (1, 2, 3, 4, 8 query heads per KV head: the forward and dQ workgroups take one,
