@@ -464,7 +464,8 @@ __device__ __forceinline__ void doc_rank(const int* __restrict__ work, int n, in
   int rank = 0;
   for (int base = 0; base < n; base += 256) {
     __syncthreads();
-    chunk[threadIdx.x] = base + threadIdx.x < n ? work[base + threadIdx.x] : -1;
+    const int at_t = base + static_cast<int>(threadIdx.x);
+    chunk[threadIdx.x] = at_t < n ? work[at_t] : -1;
     __syncthreads();
     // (entries past n hold -1: never in front of an entry, whose count is >= 0)
     const int4* chunk4 = reinterpret_cast<const int4*>(chunk);

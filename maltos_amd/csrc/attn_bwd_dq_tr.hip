@@ -191,14 +191,9 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
     lse_raw = p.lse[stat_off];
     if (!fold_stats) delta = bp.delta[stat_off];
   }
-  int qpos = 0, qseq = -1;
   int4 wq_stats = make_int4(0, -1, 0, -1);
   int4 bq_stats[BM / 64];
   if (MODE == MLTS_MASK_DOC) {
-    if (qrow < p.Sq) {
-      qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qrow];
-      qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qrow];
-    }
 #pragma unroll
     for (int w = 0; w < BM / 64; ++w) {
       const int t = (q0 >> 6) + w;

@@ -138,14 +138,9 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
   const bf16_t* V = static_cast<const bf16_t*>(p.v) + b * p.vs[0] + hkv * p.vs[1];
   bf16_t* O = static_cast<bf16_t*>(p.o) + b * p.os[0] + hq * p.os[1];
 
-  int qpos = 0, qseq = -1;
   int4 wq_stats = make_int4(0, -1, 0, -1);
   int4 bq_stats[BM / 64];
   if (MODE == MLTS_MASK_DOC) {
-    if (qrow < p.Sq) {
-      qpos = p.q_pos[static_cast<int64_t>(b) * p.Sq + qrow];
-      qseq = p.q_seq[static_cast<int64_t>(b) * p.Sq + qrow];
-    }
 #pragma unroll
     for (int w = 0; w < BM / 64; ++w) {
       const int t = (q0 >> 6) + w;
