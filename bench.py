@@ -215,6 +215,32 @@ def bench_cfg3_packed_gqa(torch, ops, _lib, dev, steps, warmup):
             "value": flops / sec / 1e12, "unit": "TFLOP/s", "frac_of_mfma_peak": flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}
 
 
+def bench_box_matrix_rate(torch, _lib, dev):
+    """What this GPU's matrix cores sustain on v_mfma_f32_32x32x16_bf16 alone (mlts_mfma_probe): on zeros, where the chip
+    holds its nominal clock, and on normally distributed operands like the attention inputs of this run, where the
+    cores' power makes it lower the clock.  The attention kernels' executed rates are fractions of the second figure."""
+    import ctypes as C
+    L = _lib.lib()
+    blocks, iters = 2048, 2000
+    out = torch.empty(blocks * 512, device=dev)
+    flops = L.mlts_mfma_probe_flops(blocks, iters)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {}
+    for label, operands in (("zeros", torch.zeros(32768, device=dev).bfloat16()),
+                            ("normal", torch.randn(32768, generator=torch.Generator().manual_seed(1234)).bfloat16().to(dev))):
+        fn = lambda: _lib.check(L.mlts_mfma_probe(operands.data_ptr(), operands.numel(), out.data_ptr(), blocks, iters, stream))
+        preheat(torch, fn)
+        _lib.kernel_timing(True)
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        ms, n = _lib.kernel_time_ms("mfma_probe")
+        _lib.kernel_timing(False)
+        res[label + "_operands_tflops"] = flops / (ms / n * 1e-3) / 1e12
+    res["workload"] = f"{blocks} workgroups x 8 wavefronts x {iters} x 16 MFMA 32x32x16 bf16, no memory traffic"
+    return res
+
+
 def bench_cfg4_ring_rank(torch, dev, steps, warmup, rank=1):
     """Configuration 4: one rank's share of zigzag ring attention at CP=4 over 32768 tokens (local Q of 8192 tokens against
     the four KV chunks, all resident; block kernels + fp32 LSE merges forward, then the backward with the global O / LSE).
@@ -607,6 +633,7 @@ def main() -> int:
                 torch.cuda.synchronize()
 
         half = max(5, args.steps // 2)
+        leg("box_matrix_rate", lambda: bench_box_matrix_rate(torch, _lib, dev))
         leg("parity_cfg2", lambda: parity_cfg2(torch, ops, dev))
         leg("attn_ds_handover_backward", lambda: bench_attention_handover(torch, ops, _lib, dev, args.steps, args.warmup))
         leg("attn_d64", lambda: bench_attention_d64(torch, ops, _lib, dev, args.steps, args.warmup))

@@ -54,6 +54,16 @@ const char* mlts_last_error(void);
 void mlts_kernel_timing_enable(int enable);
 int mlts_kernel_timing_read(const char* name, double* total_ms, int64_t* launches);
 
+/* Measurement aid with no counterpart in the reference: the rate of the matrix cores alone on this GPU.  Launches
+ * `blocks` workgroups (512 lanes, two wavefronts per SIMD) that each run `iters` x 16 v_mfma_f32_32x32x16_bf16 per
+ * wavefront on operands taken from `operands` (at least 32768 bf16, 16-byte aligned; the values set the cores' power
+ * and so the clock the chip holds: zeros reach the nominal peak, normally distributed values do not) and write one
+ * float per lane to `out` (blocks * 512 floats).  mlts_mfma_probe_flops gives the flops of such a launch; its duration
+ * is read with mlts_kernel_timing_read("mfma_probe"). */
+int64_t mlts_mfma_probe_flops(int32_t blocks, int32_t iters);
+int mlts_mfma_probe(const void* operands, int64_t n_operands, float* out, int32_t blocks, int32_t iters,
+                    mlts_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Attention                                                                                  */
 /* ------------------------------------------------------------------------------------------ */
