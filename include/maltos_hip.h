@@ -48,7 +48,8 @@ const char* mlts_last_error(void);
 /* Measurement aid with no counterpart in the reference (it times whole steps with a device
  * synchronise, tools/profile_train_perf.py:900-919): when enabled, the main kernel of each entry
  * point is bracketed by HIP events on its launch stream.  Names: "attn_fwd", "attn_bwd_dkdv",
- * "attn_bwd_dq", "adamw", "ce", "rmsnorm_fwd", "rmsnorm_bwd", "grad_to_f32".
+ * "attn_bwd_dq", "attn_bwd_dq_ds", "attn_delta", "attn_doc_prepass", "attn_merge", "adamw", "ce", "rmsnorm_fwd",
+ * "rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "grad_to_f32", "grad_sum_slices", "mfma_probe".
  * mlts_kernel_timing_read synchronises on the recorded events and returns the summed kernel time
  * and the number of launches since timing was enabled.  Enabling or disabling clears the records. */
 void mlts_kernel_timing_enable(int enable);
