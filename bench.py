@@ -27,10 +27,10 @@ PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
 
 
 def measured_hbm_traffic():
-    """HBM bytes per launch of each attention kernel on the headline workload: profiles/attn_cfg2_hbm_traffic.json, which
-    `python -m maltos_amd.profile_summary traffic` writes from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then
-    WRITE_SIZE, each scaled by the same counter over the --calibrate-traffic kernel).  Counters cannot be read from
-    inside the timed run; a missing file gives null figures."""
+    """HBM bytes per launch of each attention kernel on the headline workload: profiles/attn_cfg2_hbm_traffic.json, the
+    figures of profiles/attn_cfg2_hbm_traffic.md (two rocprofv3 --pmc runs of this script, FETCH_SIZE, then WRITE_SIZE,
+    each scaled by the same counter over the --calibrate-traffic kernel).  Counters cannot be read from inside the timed
+    run; a missing file gives null figures."""
     try:
         with open(os.path.join(PROFILES, "attn_cfg2_hbm_traffic.json")) as f:
             return {k: v["hbm_bytes_per_launch"] for k, v in json.load(f)["kernels"].items()}
@@ -58,6 +58,7 @@ def attention_inputs(torch, dev, B, H, S, D, seed=1234):
 
 
 PREHEAT_S = 0.25
+LLAMA_PREHEAT_STEPS = 25  # untimed training steps in front of the warm-up steps of the LLaMA legs
 
 
 def preheat(torch, fn, seconds=PREHEAT_S):
@@ -71,14 +72,21 @@ def preheat(torch, fn, seconds=PREHEAT_S):
         torch.cuda.synchronize()
 
 
-def timed(torch, fn, steps, warmup):
+def timed(torch, fn, steps, warmup, preheat_steps=None):
     """Mean seconds per call.  The interpreter's cyclic garbage collector is held off during the timed calls (as
-    timeit does): one full collection is a 50-100 ms pause, which in a launch-bound loop of ten steps is the result."""
+    timeit does): one full collection is a 50-100 ms pause, which in a launch-bound loop of ten steps is the result.
+    preheat_steps: a fixed number of untimed calls in place of the wall-time pre-heat, for steps that change state
+    (training steps: legs that are compared afterwards must have taken the same number of optimizer steps)."""
     import gc
     gc.collect()  # before the pre-heat: a collection behind it would leave the GPU idle long enough to drop its clocks
     gc.disable()
     try:
-        preheat(torch, fn)
+        if preheat_steps is None:
+            preheat(torch, fn)
+        else:
+            for _ in range(preheat_steps):
+                fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -113,7 +121,7 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(4, 16, 4096, 12
     torch.cuda.synchronize()
     sec = (time.perf_counter() - t0) / steps
     kernels = {}
-    for name in ("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq", "attn_bwd_dq_ds"):
+    for name in ("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"):
         total_ms, launches = _lib.kernel_time_ms(name)
         if launches:
             kernels[name] = {"ms": total_ms / launches, "launches_per_step": launches / steps}
@@ -121,15 +129,8 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(4, 16, 4096, 12
     _lib.kernel_timing(False)
     # algorithmic flops per launch of each kernel (FlashAttention convention: 2 GEMMs forward, 5 backward: S, dP, dV,
     # dK, dQ, each fwd_flops / 2)
-    kernel_flops = {"attn_fwd": fwd_flops}
-    if "attn_bwd_dq_ds" in kernels:  # dK/dV kernel hands dS over: it runs S, dP, dV, dK, the dQ kernel only dQ
-        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops * 0.8
-        kernel_flops["attn_bwd_dq_ds"] = 2.5 * fwd_flops * 0.2
-    elif "attn_bwd_dq" in kernels:  # both kernels recompute S and dP; credited 3 : 2 (dV, dK, + S | dQ, + dP)
-        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops * 0.6
-        kernel_flops["attn_bwd_dq"] = 2.5 * fwd_flops * 0.4
-    else:
-        kernel_flops["attn_bwd_dkdv"] = 2.5 * fwd_flops
+    # both backward kernels recompute S and dP; the five conventional products are credited 3 : 2 (dV, dK, + S | dQ, + dP)
+    kernel_flops = {"attn_fwd": fwd_flops, "attn_bwd_dkdv": 2.5 * fwd_flops * 0.6, "attn_bwd_dq": 2.5 * fwd_flops * 0.4}
     for name, rec in kernels.items():
         rec["tflops"] = kernel_flops[name] / (rec["ms"] * 1e-3) / 1e12
     # the row-wise delta = sum(dO * O) pass in front of the backward kernels: memory bound, reads dO and O once
@@ -139,19 +140,6 @@ def bench_attention(torch, ops, _lib, dev, steps, warmup, shape=(4, 16, 4096, 12
         kernels["attn_delta"] = {"ms": total_ms / launches, "launches_per_step": launches / steps,
                                  "gbps": nbytes / (total_ms / launches * 1e-3) / 1e9}
     return sec, flops, kernels, kernel_flops
-
-
-def bench_attention_handover(torch, ops, _lib, dev, steps, warmup):
-    """The same attention step with the dS hand-over allowed (ops.set_backward_ds_handover_limit): the dK/dV kernel
-    stores dS (2 bytes per score, 2.1 GB of workspace at this shape) and the dQ kernel reads it instead of recomputing
-    S and dP.  The default backward recomputes and keeps the workspace O(B * H * S)."""
-    previous = ops.set_backward_ds_handover_limit(4 << 30)
-    try:
-        sec, flops, kernels, _ = bench_attention(torch, ops, _lib, dev, steps, warmup)
-    finally:
-        ops.set_backward_ds_handover_limit(previous)
-    return {"value": (flops["fwd"] + flops["bwd"]) / sec / 1e12, "unit": "TFLOP/s", "ms_per_step": sec * 1e3,
-            "kernels": kernels, "workspace_bytes": 2 * 4 * 16 * 4096 * 4096}
 
 
 def bench_attention_d64(torch, ops, _lib, dev, steps, warmup):
@@ -215,32 +203,6 @@ def bench_cfg3_packed_gqa(torch, ops, _lib, dev, steps, warmup):
             "value": flops / sec / 1e12, "unit": "TFLOP/s", "frac_of_mfma_peak": flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS}
 
 
-def bench_box_matrix_rate(torch, _lib, dev):
-    """What this GPU's matrix cores sustain on v_mfma_f32_32x32x16_bf16 alone (mlts_mfma_probe): on zeros, where the chip
-    holds its nominal clock, and on normally distributed operands like the attention inputs of this run, where the
-    cores' power makes it lower the clock.  The attention kernels' executed rates are fractions of the second figure."""
-    import ctypes as C
-    L = _lib.lib()
-    blocks, iters = 2048, 2000
-    out = torch.empty(blocks * 512, device=dev)
-    flops = L.mlts_mfma_probe_flops(blocks, iters)
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    res = {}
-    for label, operands in (("zeros", torch.zeros(32768, device=dev).bfloat16()),
-                            ("normal", torch.randn(32768, generator=torch.Generator().manual_seed(1234)).bfloat16().to(dev))):
-        fn = lambda: _lib.check(L.mlts_mfma_probe(operands.data_ptr(), operands.numel(), out.data_ptr(), blocks, iters, stream))
-        preheat(torch, fn)
-        _lib.kernel_timing(True)
-        for _ in range(5):
-            fn()
-        torch.cuda.synchronize()
-        ms, n = _lib.kernel_time_ms("mfma_probe")
-        _lib.kernel_timing(False)
-        res[label + "_operands_tflops"] = flops / (ms / n * 1e-3) / 1e12
-    res["workload"] = f"{blocks} workgroups x 8 wavefronts x {iters} x 16 MFMA 32x32x16 bf16, no memory traffic"
-    return res
-
-
 def bench_cfg4_ring_rank(torch, dev, steps, warmup, rank=1):
     """Configuration 4: one rank's share of zigzag ring attention at CP=4 over 32768 tokens (local Q of 8192 tokens against
     the four KV chunks, all resident; block kernels + fp32 LSE merges forward, then the backward with the global O / LSE).
@@ -299,6 +261,88 @@ def parity_cfg2(torch, ops, dev):
     out["reference"] = "torch SDPA math backend in fp32 on the bf16-rounded inputs, batch element 0 of configuration 2"
     out["bound"] = "2e-2 max-abs (O, dQ, dK, dV), 2e-3 (LSE)"
     return out
+
+
+def _parity_update(out, name, got, ref):
+    err = (got.float() - ref.float()).abs().max().item()
+    rec = out.setdefault(name, {"max_abs": 0.0, "largest_value": 0.0})
+    rec["max_abs"] = max(rec["max_abs"], err)
+    rec["largest_value"] = max(rec["largest_value"], ref.float().abs().max().item())
+
+
+def _parity_finish(out, reference, bound):
+    for rec in out.values():
+        rec["rel"] = rec["max_abs"] / rec.pop("largest_value")
+    out["reference"] = reference
+    out["bound"] = bound
+    return out
+
+
+def parity_cfg3(torch, ops, dev):
+    """Largest differences of O, LSE, dQ, dK, dV of configuration 3 (first batch row, every document, all heads) against
+    the oracle: causal attention of each document alone in fp32, differentiated by autograd, on the GPU tensors."""
+    from oracle import attention as oa
+
+    B, S, Hq, Hkv, D = 1, 8192, 32, 8, 128
+    gen = torch.Generator().manual_seed(1234)
+    pos, seq, _ = packed_rows(torch, B, S, gen)
+    q = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    k = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    v = torch.randn(B, Hkv, S, D, generator=gen).bfloat16().to(dev)
+    do = torch.randn(B, Hq, S, D, generator=gen).bfloat16().to(dev)
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ids = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+    o, lse = ops.attention(qg, kg, vg, mask_mode=ops.MASK_DOC, return_lse=True, **ids)
+    o.backward(do)
+    out = {}
+    starts = (seq[0, 1:] != seq[0, :-1]).nonzero().flatten().add(1).tolist()
+    for a, b in zip([0] + starts, starts + [S]):
+        sl = slice(a, b)
+        qf, kf, vf = (t[:, :, sl].float().requires_grad_(True) for t in (q, k, v))
+        want_o, want_lse = oa.attention_with_lse(qf, kf, vf, oa.causal_mask(b - a, b - a, dev))
+        want_o.backward(do[:, :, sl].float())
+        for name, got, ref in (("O", o[:, :, sl], want_o), ("LSE", lse[:, :, sl], want_lse), ("dQ", qg.grad[:, :, sl], qf.grad),
+                               ("dK", kg.grad[:, :, sl], kf.grad), ("dV", vg.grad[:, :, sl], vf.grad)):
+            _parity_update(out, name, got, ref.detach())
+    return _parity_finish(out, "oracle.attention (fp32) per document on the bf16-rounded inputs, batch row 0 of configuration 3's shapes, "
+                               f"{len(starts) + 1} documents",
+                          "2e-2 + 2^-8 |value| (O, dQ, dK, dV; dK and dV are sums over four query heads, their half ulp exceeds 2e-2 "
+                          "where |value| > 5), 2e-3 (LSE)")
+
+
+def parity_cfg4(torch, dev, rank=1, heads=(0, 15)):
+    """Largest differences of O, LSE, dQ and the four chunks' dK, dV of configuration 4 (one rank's ring share) against
+    the oracle: ONE pass of causal attention over all 32768 tokens in fp32 with dO zero outside the rank, on `heads`."""
+    from maltos_amd.ring_attention import zigzag_ring_attention
+    from maltos_amd.ring_layout import expected_zigzag_ring_positions
+    from oracle import attention as oa
+
+    W, H, S_loc, D = 4, 16, 8192, 128
+    total = W * S_loc
+    gen = torch.Generator().manual_seed(1234)
+    gq, gk, gv, gdo = (torch.randn(1, H, total, D, generator=gen).bfloat16().to(dev) for _ in range(4))
+    pos = [expected_zigzag_ring_positions(S_loc, rank=r, world_size=W, device=dev) for r in range(W)]
+    q = gq.index_select(2, pos[rank]).requires_grad_(True)
+    chunks = [(gk.index_select(2, p_).requires_grad_(True), gv.index_select(2, p_).requires_grad_(True)) for p_ in pos]
+    o, lse = zigzag_ring_attention(q, chunks, rank=rank, world_size=W, return_lse=True)
+    o.backward(gdo.index_select(2, pos[rank]))
+    do_masked = torch.zeros_like(gdo)
+    do_masked[:, :, pos[rank]] = gdo[:, :, pos[rank]]
+    mask = oa.causal_mask(total, total, dev)
+    out = {}
+    for h in heads:
+        qf, kf, vf = (t[:, h:h + 1].float().requires_grad_(True) for t in (gq, gk, gv))
+        want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
+        want_o.backward(do_masked[:, h:h + 1].float())
+        _parity_update(out, "O", o[:, h:h + 1], want_o.detach()[:, :, pos[rank]])
+        _parity_update(out, "LSE", lse[:, h:h + 1], want_lse.detach()[:, :, pos[rank]])
+        _parity_update(out, "dQ", q.grad[:, h:h + 1], qf.grad[:, :, pos[rank]])
+        for src, (kc, vc) in enumerate(chunks):
+            _parity_update(out, "dK", kc.grad[:, h:h + 1], kf.grad[:, :, pos[src]])
+            _parity_update(out, "dV", vc.grad[:, h:h + 1], vf.grad[:, :, pos[src]])
+        del qf, kf, vf, want_o, want_lse
+    return _parity_finish(out, f"oracle.attention (fp32): one causal pass over all 32768 tokens, rank {rank}, heads {list(heads)}",
+                          "2e-2 max-abs (O, dQ, dK, dV), 2e-3 (LSE)")
 
 
 def bench_adamw(torch, ops, _lib, dev, steps, warmup):
@@ -451,10 +495,13 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False):
         out["norm"] = z.step(1.0)
         out["loss"] = loss
 
-    sec = timed(torch, step_zero1 if zero1 else step_graph if graph else step, steps, warmup)
+    # a fixed number of untimed steps (~0.3 s) in front: the three legs then report loss and gradient norm of the same
+    # optimizer step, and they agree when the layouts compute the same thing
+    sec = timed(torch, step_zero1 if zero1 else step_graph if graph else step, steps, warmup, preheat_steps=LLAMA_PREHEAT_STEPS)
     tokens = 8 * 2048
     res = {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"].detach()),
            "grad_norm_last": float(out["norm"]) if zero1 else float(out["sq"].sqrt()),
+           "optimizer_steps_taken": LLAMA_PREHEAT_STEPS + warmup + steps,
            "params": sum(p.numel() for p in model.parameters()),
            "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12}
     if zero1:
@@ -520,8 +567,8 @@ def cpu_baseline_llama(torch, dev, which):
     """One full train step (forward, backward, clip for configuration 5, stock AdamW on fp32 masters) of the CPU oracle
     on the host cores at full size, next to the same first step through the HIP path from identical weights and
     tokens: time, tokens/s and the parity of loss and gradient norm."""
-    from maltos_amd.grad_clip import clip_grad_norm_
-    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+    from maltos_amd.grad_clip import clip_grad_norm_, clip_grad_norm_fused_
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
     from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
     from oracle import llama as ol
 
@@ -542,29 +589,35 @@ def cpu_baseline_llama(torch, dev, which):
         for n, p in model.named_parameters():
             p.copy_(params[n])
     model = model.to(dtype)
+    if dtype != torch.float32:
+        set_grad_accumulation_into_buffers(model)   # as the llama50m_train_step leg: dW adds into the flat gradient buffer
     adam = lambda ps: FusedAdamW(ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
     opt = MasterWeightsOptimizer(model.parameters(), optimizer_factory=adam) if dtype != torch.float32 else adam(model.parameters())
     data = {"input_ids": inp.to(dev), "labels": lab.to(dev)}
     first = {}
 
-    def step():
+    def step(timed_step=True):
         loss = model(data)
         loss.backward()
-        norm = clip_grad_norm_(opt, max_norm if max_norm is not None else float("inf"))   # inf: the norm only
+        if not timed_step:   # the first step: the norm is read back for the parity figures (one host round trip)
+            first["norm"] = float(clip_grad_norm_(opt, max_norm if max_norm is not None else float("inf")))   # inf: the norm only
+            first["loss"] = float(loss.detach())
+        elif max_norm is not None:   # the timed steps clip on the device, as the llama50m_train_step leg does
+            clip_grad_norm_fused_(opt, max_norm)
         opt.step()
         opt.zero_grad(set_to_none=True)
-        first.setdefault("loss", float(loss.detach()))
-        first.setdefault("norm", float(norm))
 
-    step()
-    gpu_sec = timed(torch, step, 10, 3)
+    step(timed_step=False)
+    gpu_sec = timed(torch, step, 10, 3, preheat_steps=LLAMA_PREHEAT_STEPS)
     tokens = batch * seq
     return {"workload": f"{'tiny LLaMA fp32 (configuration 1)' if which == 'cfg1' else 'LLaMA-50M bf16 (configuration 5)'} full train step, "
                         f"batch {batch} x {seq}",
             "cpu": {"ms": cpu_sec * 1e3, "tokens_per_sec": tokens / cpu_sec, "cores": torch.get_num_threads(), "kind": "port",
                     "sample": f"oracle.llama.train_step (fp32 PyTorch restatement, stock AdamW) at full size, {timed_steps} timed step(s)"
                               + (", 1 warm-up" if which == "cfg1" else ", no warm-up")},
-            "gpu": {"ms": gpu_sec * 1e3, "tokens_per_sec": tokens / gpu_sec},
+            "gpu": {"ms": gpu_sec * 1e3, "tokens_per_sec": tokens / gpu_sec,
+                    "clip": "none (the configuration has no clip)" if max_norm is None else
+                            "global-norm clip at 1.0 applied on the device (no host read): the eager step of extra.llama50m_train_step"},
             "parity": {"loss": {"hip": first["loss"], "oracle": want_loss, "rel": abs(first["loss"] - want_loss) / abs(want_loss)},
                        "grad_norm": {"hip": first["norm"], "oracle": want_norm, "rel": abs(first["norm"] - want_norm) / abs(want_norm)},
                        "bound": "1e-4 relative (fp32)" if which == "cfg1" else "1e-3 relative (bf16)"}}
@@ -633,12 +686,12 @@ def main() -> int:
                 torch.cuda.synchronize()
 
         half = max(5, args.steps // 2)
-        leg("box_matrix_rate", lambda: bench_box_matrix_rate(torch, _lib, dev))
         leg("parity_cfg2", lambda: parity_cfg2(torch, ops, dev))
-        leg("attn_ds_handover_backward", lambda: bench_attention_handover(torch, ops, _lib, dev, args.steps, args.warmup))
         leg("attn_d64", lambda: bench_attention_d64(torch, ops, _lib, dev, args.steps, args.warmup))
         leg("cfg3_packed_gqa", lambda: bench_cfg3_packed_gqa(torch, ops, _lib, dev, half, args.warmup))
+        leg("parity_cfg3", lambda: parity_cfg3(torch, ops, dev))
         leg("cfg4_ring_rank", lambda: bench_cfg4_ring_rank(torch, dev, half, 3))
+        leg("parity_cfg4", lambda: parity_cfg4(torch, dev))
         leg("adamw_flat_fp32", lambda: bench_adamw(torch, ops, _lib, dev, max(10, args.steps), args.warmup))
         leg("hbm_kernels", lambda: bench_hbm_kernels(torch, ops, _lib, dev))
         leg("llama50m_train_step", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup)))

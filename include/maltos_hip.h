@@ -48,22 +48,12 @@ const char* mlts_last_error(void);
 /* Measurement aid with no counterpart in the reference (it times whole steps with a device
  * synchronise, tools/profile_train_perf.py:900-919): when enabled, the main kernel of each entry
  * point is bracketed by HIP events on its launch stream.  Names: "attn_fwd", "attn_bwd_dkdv",
- * "attn_bwd_dq", "attn_bwd_dq_ds", "attn_delta", "attn_doc_prepass", "attn_merge", "adamw", "ce", "rmsnorm_fwd",
- * "rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "grad_to_f32", "grad_sum_slices", "mfma_probe".
+ * "attn_bwd_dq", "attn_delta", "attn_doc_prepass", "attn_merge", "adamw", "ce", "rmsnorm_fwd",
+ * "rmsnorm_bwd", "rope", "swiglu_fwd", "swiglu_bwd", "grad_to_f32", "grad_sum_slices".
  * mlts_kernel_timing_read synchronises on the recorded events and returns the summed kernel time
  * and the number of launches since timing was enabled.  Enabling or disabling clears the records. */
 void mlts_kernel_timing_enable(int enable);
 int mlts_kernel_timing_read(const char* name, double* total_ms, int64_t* launches);
-
-/* Measurement aid with no counterpart in the reference: the rate of the matrix cores alone on this GPU.  Launches
- * `blocks` workgroups (512 lanes, two wavefronts per SIMD) that each run `iters` x 16 v_mfma_f32_32x32x16_bf16 per
- * wavefront on operands taken from `operands` (at least 32768 bf16, 16-byte aligned; the values set the cores' power
- * and so the clock the chip holds: zeros reach the nominal peak, normally distributed values do not) and write one
- * float per lane to `out` (blocks * 512 floats).  mlts_mfma_probe_flops gives the flops of such a launch; its duration
- * is read with mlts_kernel_timing_read("mfma_probe"). */
-int64_t mlts_mfma_probe_flops(int32_t blocks, int32_t iters);
-int mlts_mfma_probe(const void* operands, int64_t n_operands, float* out, int32_t blocks, int32_t iters,
-                    mlts_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------ */
 /* Attention                                                                                  */
@@ -114,13 +104,6 @@ int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int accumulate_f
  * (runtime/layers/flash_utils.py:566-640).  Returns 0 bytes / does nothing for shapes the generic kernels serve. */
 int64_t mlts_attn_doc_plan_bytes(const mlts_attn_shape* s);
 int mlts_attn_doc_plan(const mlts_attn_shape* s, void* plan, int64_t plan_bytes, mlts_stream_t stream);
-
-/* Optional trade of memory for matrix work in mlts_attn_bwd: when the caller's workspace is at least
- * mlts_attn_bwd_workspace_bytes + mlts_attn_bwd_ds_handover_bytes, the dK/dV kernel hands dS (bf16, 2 bytes per
- * (query, key) pair: 2 * B * Hq * Sq * Sk bytes) to the dQ kernel instead of the dQ kernel recomputing the scores.
- * Returns 0 for calls the hand-over does not serve (head_dim other than 128, MLTS_MASK_DOC, fp32 accumulation).
- * With a smaller workspace the backward recomputes; results differ only in the rounding of dS. */
-int64_t mlts_attn_bwd_ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32);
 
 /* O = softmax(scale * Q K^T + mask) V and LSE = logsumexp (natural log, fp32, [B, Hq, Sq]).
  * Replaces F.scaled_dot_product_attention (utils/attention_backend.py:60-64,109-116),

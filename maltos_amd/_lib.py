@@ -66,13 +66,10 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     "mlts_kernel_timing_enable": (None, [C.c_int]),
     "mlts_kernel_timing_read": (C.c_int, [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]),
     "mlts_attn_supports": (C.c_char_p, [_SHAPE_P]),
-    "mlts_mfma_probe_flops": (C.c_int64, [C.c_int32, C.c_int32]),
-    "mlts_mfma_probe": (C.c_int, [_P, C.c_int64, _P, C.c_int32, C.c_int32, _P]),
     "mlts_attn_doc_plan_bytes": (C.c_int64, [_SHAPE_P]),
     "mlts_attn_doc_plan": (C.c_int, [_SHAPE_P, _P, C.c_int64, _P]),
     "mlts_attn_fwd_workspace_bytes": (C.c_int64, [_SHAPE_P]),
     "mlts_attn_bwd_workspace_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
-    "mlts_attn_bwd_ds_handover_bytes": (C.c_int64, [_SHAPE_P, C.c_int]),
     "mlts_attn_fwd": (C.c_int, [_SHAPE_P, _P, _P, _P, _P, _P, _P, C.c_int64, _P]),
     "mlts_attn_bwd": (
         C.c_int,

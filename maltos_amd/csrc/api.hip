@@ -78,5 +78,5 @@ int mlts_check_launch(const char* what) {
   return MLTS_OK;
 }
 
-extern "C" int mlts_abi_version(void) { return 3; }
+extern "C" int mlts_abi_version(void) { return 4; }
 extern "C" const char* mlts_last_error(void) { return g_error; }

@@ -9,8 +9,6 @@ int mlts_attn_fwd_bf16_dma(const AttnParams& p, int D, int mode, hipStream_t st)
 int64_t mlts_attn_bwd_dkdv_split_workspace(int64_t B, int64_t Hq, int64_t Sq);                             // attn_bwd_split.hip
 int mlts_attn_bwd_dkdv_bf16_split(AttnBwdParams bp, int D, int mode, void* workspace, bool lse2_ready, hipStream_t st);    // attn_bwd_split.hip
 int mlts_attn_bwd_dq_bf16_tr(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_tr.hip
-int64_t mlts_attn_bwd_ds_bytes(int64_t B, int64_t Hq, int64_t Sq, int64_t Sk);                              // attn_bwd_dq_ds.hip
-int mlts_attn_bwd_dq_bf16_ds(const AttnBwdParams& bp, int D, int mode, hipStream_t st);                    // attn_bwd_dq_ds.hip
 int mlts_attn_generic_fwd(const AttnParams& p, int D, int dtype, int mode, hipStream_t st);
 int mlts_attn_generic_bwd(const AttnBwdParams& bp, int D, int dtype, int mode, hipStream_t st);
 int mlts_attn_delta(const void* dout, const int64_t* dos, const void* o, const int64_t* os, float* delta, int B, int H,
@@ -160,35 +158,17 @@ __global__ __launch_bounds__(256) void merge_kernel(float* __restrict__ out_acc,
 }
 
 
-// whether the dK/dV kernel may hand -dS to the dQ kernel for this call: head_dim 128 without a document mask and with
-// gradients in the input dtype (head_dim 64 has half the matrix work per pair and the same hand-over bytes, so
-// recomputing is faster there; gradients accumulated in fp32, the ring steps, keep the recomputed, once-rounded dS)
-int64_t ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32) {
-  if (!uses_mfma(s) || s->mask_mode == MLTS_MASK_DOC || s->D != 128 || accumulate_f32 || s->Sq == 0 || s->Sk == 0 || s->B == 0)
-    return 0;
-  return mlts_attn_bwd_ds_bytes(s->B, s->Hq, s->Sq, s->Sk);
-}
-
 int64_t bwd_min_workspace(const mlts_attn_shape* s) {
   const int64_t delta = align256(static_cast<int64_t>(s->B) * s->Hq * s->Sq * 4);
   const int64_t lse2 = uses_mfma(s) ? mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq) : 0;
   return stats_bytes(s, true) + delta + lse2;
 }
 
-// Default: the recomputing dQ kernel first, which also writes the row statistics (delta, lse2) into the workspace, then
-// the dK/dV kernel that reads them.  With a dS hand-over (ds_ws): statistics passes, dK/dV kernel, dQ from its dS.
-int attn_bwd_bf16(AttnBwdParams bp, int D, int mode, float* delta_ws, void* lse2_ws, void* ds_ws, bool stats_in_dq,
-                  hipStream_t st) {
+// The recomputing dQ kernel first, which (stats_in_dq) also writes the row statistics (delta, lse2) into the workspace,
+// then the dK/dV kernel that reads them.
+int attn_bwd_bf16(AttnBwdParams bp, int D, int mode, float* delta_ws, void* lse2_ws, bool stats_in_dq, hipStream_t st) {
   const AttnParams& p = bp.a;
   bp.nkt = (p.Sk + 127) / 128;
-  if (ds_ws) {
-    bp.ds_ws = ds_ws;
-    bp.ds_nkb = (p.Sk + 31) / 32;
-    bp.ds_nqt = (p.Sq + 63) / 64;
-    int rc = mlts_attn_bwd_dkdv_bf16_split(bp, D, mode, lse2_ws, false, st);
-    if (rc != MLTS_OK) return rc;
-    return mlts_attn_bwd_dq_bf16_ds(bp, D, mode, st);
-  }
   if (stats_in_dq) {
     bp.delta_out = delta_ws;
     bp.lse2_out = static_cast<float*>(lse2_ws);
@@ -226,8 +206,6 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
   }
   bp.accumulate_f32 = accumulate_f32 ? 1 : 0;
   bp.nkt = 0;
-  bp.ds_ws = nullptr;
-  bp.ds_nkb = bp.ds_nqt = 0;
   bp.delta_out = bp.lse2_out = nullptr;
   if (uses_mfma(s)) {
     MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
@@ -240,20 +218,14 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
     MLTS_REQUIRE(do_stride[2] < kMaxRowStride, "%s: the sequence stride of dout must be below 2^24 elements", who);
   }
   void* lse2_ws = ws;
-  void* ds_ws = nullptr;
-  if (uses_mfma(s)) {
-    ws += mlts_attn_bwd_dkdv_split_workspace(s->B, s->Hq, s->Sq);
-    const int64_t ds_bytes = ds_handover_bytes(s, accumulate_f32);
-    if (ds_bytes > 0 && workspace_bytes >= need + ds_bytes) ds_ws = ws;
-  }
   // the recomputing dQ kernel forms delta itself from 16-byte chunks of the O rows
-  const bool stats_in_dq = uses_mfma(s) && !ds_ws && s->Sk > 0 && mlts_aligned16(o) && strides_aligned(s->o_stride, 2);
+  const bool stats_in_dq = uses_mfma(s) && s->Sk > 0 && mlts_aligned16(o) && strides_aligned(s->o_stride, 2);
   if (s->Sq > 0 && !stats_in_dq) {
     int rc = mlts_attn_delta(dout, do_stride, o, s->o_stride, delta, s->B, s->Hq, s->Sq, s->D, s->dtype, st);
     if (rc != MLTS_OK) return rc;
   }
   if (!uses_mfma(s)) return mlts_attn_generic_bwd(bp, s->D, s->dtype, s->mask_mode, st);
-  return attn_bwd_bf16(bp, s->D, s->mask_mode, delta, lse2_ws, ds_ws, stats_in_dq, st);
+  return attn_bwd_bf16(bp, s->D, s->mask_mode, delta, lse2_ws, stats_in_dq, st);
 }
 
 // ---- scratch of the entry point that allocates nothing --------------------------------------------------------
@@ -598,11 +570,6 @@ extern "C" int64_t mlts_attn_bwd_workspace_bytes(const mlts_attn_shape* s, int a
   return bwd_min_workspace(s);
 }
 
-extern "C" int64_t mlts_attn_bwd_ds_handover_bytes(const mlts_attn_shape* s, int accumulate_f32) {
-  if (shape_problem(s)) return -1;
-  return ds_handover_bytes(s, accumulate_f32);
-}
-
 extern "C" int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void* k, const void* v, void* o, float* lse,
                              void* workspace, int64_t workspace_bytes, mlts_stream_t stream) {
   const char* why = shape_problem(s);
@@ -652,7 +619,6 @@ extern "C" int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout,
   void* ws = nullptr;
   int rc = scratch_for_current_device(&ws);
   if (rc != MLTS_OK) return rc;
-  // exactly `need` bytes are offered, so the dS hand-over (which needs more) is never taken
   return attn_bwd_impl("mlts_attn_bwd_noalloc", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv,
                        dv_stride, accumulate_f32, ws, need, static_cast<hipStream_t>(stream));
 }

@@ -1,8 +1,7 @@
 // Attention backward, dK and dV, head_dim 64 and 128, bf16: two-role workgroup.
 //
 // A workgroup owns 128 keys of one (batch, kv head) and walks the 64-row query tiles that can see them (all
-// query heads of the GQA group), as attn_bwd.hip does, but its EIGHT wavefronts come in two roles per 32-key
-// block kb = wave % 4:
+// query heads of the GQA group); its EIGHT wavefronts come in two roles per 32-key block kb = wave % 4:
 //     role 0 (wave < 4):   S = Q K^T,  P = exp2(S c - lse2)  ->  dV += P^T dO      and hands P (bf16) over in LDS
 //     role 1 (wave >= 4):  delta - dO V^T,  -dS = P (delta - dO V^T)  ->  -dK += (-dS)^T Q     one tile behind
 //                          (per barrier interval: dS of tile k-1, dP of tile k, then the dK products of tile k-1)
@@ -615,20 +614,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
       }
     }
   };
-  // hand -dS of tile x over to the dQ kernel: four fully coalesced 1 KiB stores per wavefront
-  auto role1_ds_store = [&](const Pos& x) {
-    if (MODE == MLTS_MASK_NONE && wkv0 + 32 > p.Sk && kj >= p.Sk) {  // without a mask, keys past the end hold garbage
-#pragma unroll
-      for (int f = 0; f < 4; ++f)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) dsfr[f][i] = static_cast<bf16_t>(0.f);
-    }
-    const int64_t blk = ((static_cast<int64_t>(b) * p.Hq + hkv * group + x.h) * bp.ds_nkb + (wkv0 >> 5)) * bp.ds_nqt + qt_begin + x.qt;
-    unsigned char* dst = static_cast<unsigned char*>(bp.ds_ws) + blk * 4096 + lane * 16;
-#pragma unroll
-    for (int f = 0; f < 4; ++f)  // streamed: the hand-over is read once, by another kernel, and must not evict Q/dO
-      __builtin_nontemporal_store(__builtin_bit_cast(v4i32, dsfr[f]), reinterpret_cast<v4i32*>(dst + f * 1024));
-  };
   // ---- ... and, after the dp of the next tile, -dK += (-dS)^T Q (transposed reads, while role 0 does its softmax) ----
   auto role1_dk = [&](const int stage) {
     const uint32_t sb = lds0 + stage * STAGE_BYTES;
@@ -676,7 +661,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     int stage = 0, k = 0;
     bool prev_active = false;
     int prev_stage = 0;
-    Pos prev_it = it;
     while (!at_end(it)) {
       const int cls = classify(it);  // before the scan of the needed tiles moves on
       const unsigned long long vis = vis_next;
@@ -698,12 +682,8 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
         if (prev_active) role1_dk(prev_stage);
       }
       if (!at_end(itn)) stage_store(stage == STAGES - 1 ? 0 : stage + 1);
-      // after the wait for the next tile's loads: loads and stores complete out of order with respect to each other,
-      // so a store in front of that wait would make it wait for the store's acknowledgement as well
-      if (ROLE == 1 && prev_active && bp.ds_ws) role1_ds_store(prev_it);
       prev_active = cls != TILE_SKIP;
       prev_stage = stage;
-      prev_it = it;
       it = itn;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
       ++k;
@@ -711,7 +691,6 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dkdv_split_kernel(const Attn
     drain_and_barrier();
     if (ROLE == 1 && prev_active) {
       role1_ds(((k - 1) & 1) * (4 * PBUF_BYTES));
-      if (bp.ds_ws) role1_ds_store(prev_it);
       role1_dk(prev_stage);
     }
     last_stage = prev_stage;

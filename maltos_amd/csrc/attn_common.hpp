@@ -63,25 +63,12 @@ struct AttnBwdParams {
   int64_t dks[3], dvs[3];
   int accumulate_f32;  // dk/dv are fp32 and added to
   int nkt;             // key tiles per (batch, kv head)
-  // Optional hand-over of -dS (bf16) from the dK/dV kernel to the dQ kernel, null when dQ recomputes it.  One 4 KiB
-  // block per (batch, query head, 32-key block, 64-query tile), [B][Hq][ds_nkb][ds_nqt]; a block is
-  // [fragment f = 0..3][lane = key + 32 hh][8 values]: value i of fragment f is query 16 f + 8 (i / 4) + 4 hh + i % 4
-  // of the tile (the A-operand order of the dK product).  Blocks that no query can see are not written.
-  void* ds_ws;
-  int ds_nkb, ds_nqt;
   // Optional outputs of the recomputing dQ kernel, which then runs first and takes the place of the separate row
   // statistics passes: delta_out[B, Hq, Sq] = rowsum(dO * O) (the kernel ignores `delta` and reads `a.o`), and
   // lse2_out[B * Hq * Sq + 1] = lse * log2(e) with +inf for rows that saw no key and in the last entry.
   float* delta_out;
   float* lse2_out;
 };
-
-// whether block (32-key block kb, 64-query tile qt) of the dS hand-over is written (MLTS_MASK_NONE / MLTS_MASK_CAUSAL)
-__host__ __device__ __forceinline__ bool mlts_ds_block_written(int kb, int qt, int Sq, int Sk, int causal_off, bool causal) {
-  if (kb * 32 >= Sk || qt * 64 >= Sq) return false;
-  const int last_q = (qt * 64 + 64 < Sq ? qt * 64 + 64 : Sq) - 1;
-  return !causal || kb * 32 <= last_q + causal_off;
-}
 
 enum TileClass { TILE_SKIP = 0, TILE_FULL = 1, TILE_MASKED = 2 };
 

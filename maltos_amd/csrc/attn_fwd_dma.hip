@@ -1,7 +1,7 @@
-// Attention forward, head_dim 64 and 128, bf16: the gfx950 memory pipeline version.
+// Attention forward, head_dim 64 and 128, bf16.
 //
-// Same math and register layouts as attn_fwd.hip (S^T = K Q^T, P in registers, O^T = V^T P^T, eight
-// wavefronts x 32 query rows), but K and V tiles travel global -> LDS with the 16-byte LDS-DMA loads
+// S^T = K Q^T, P in registers, O^T = V^T P^T, eight wavefronts x 32 query rows; K and V tiles travel
+// global -> LDS with the 16-byte LDS-DMA loads
 // (global_load_lds_dwordx4: no staging registers, no ds_write, no VALU work) into a four-stage ring, so a
 // tile's loads are issued two tiles ahead of its use.  Tiles are stored row major; V^T fragments come from
 // ds_read_b64_tr_b16 (transpose-on-read), so nothing is transposed on the way in.

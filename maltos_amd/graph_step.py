@@ -67,7 +67,8 @@ class CapturedForwardBackward:
             loss.backward()
             return loss
 
-        # warm-up on a side stream (workspaces, lazily created module state, library handles), then record
+        # warm-up on a side stream (workspaces, lazily created module state, library handles), then record on the SAME
+        # stream: autograd ties each parameter's gradient accumulator to the stream of the forward pass that created it
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -77,7 +78,7 @@ class CapturedForwardBackward:
         torch.cuda.synchronize()
         self._check_grads_in_place()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        with torch.cuda.graph(self.graph, stream=side):
             self.loss = forward_backward()
         self._check_grads_in_place()
         clear()            # the warm-up passes ran for real; recording itself executes nothing

@@ -19,7 +19,6 @@ from ._lib import MASK_CAUSAL, MASK_DOC, MASK_NONE, MLTS_BF16, MLTS_F32, AttnSha
 __all__ = [
     "MASK_NONE", "MASK_CAUSAL", "MASK_DOC",
     "attention", "attention_forward", "attention_backward", "attention_backward_accumulate", "attention_merge_",
-    "set_backward_ds_handover_limit",
     "rms_norm", "rope", "rope_pair", "swiglu", "cross_entropy",
     "adamw_step_", "sq_norm", "scale_", "grad_to_f32_",
 ]
@@ -192,22 +191,6 @@ def attention_forward(q, k, v, *, mask_mode: int, scale: float | None = None, q_
     return o, lse
 
 
-# Largest dS hand-over workspace (bytes) attention_backward may allocate on top of the O(S) one; 0 = always recompute.
-_BWD_DS_HANDOVER_MAX_BYTES = 0
-
-
-def set_backward_ds_handover_limit(max_bytes: int) -> int:
-    """Lets the head_dim-128 backward trade memory for matrix work: calls whose dS hand-over (2 * B * Hq * Sq * Sk
-    bytes) fits `max_bytes` allocate it, and the dQ kernel then reads dS from the dK/dV kernel instead of recomputing
-    the scores.  0 (the default) keeps the workspace O(B * Hq * Sq) like the flash backward the reference calls
-    (runtime/layers/flash_utils.py:239-258).  Returns the previous limit."""
-    global _BWD_DS_HANDOVER_MAX_BYTES
-    if max_bytes < 0:
-        raise ValueError("the hand-over limit is a byte count >= 0")
-    previous, _BWD_DS_HANDOVER_MAX_BYTES = _BWD_DS_HANDOVER_MAX_BYTES, int(max_bytes)
-    return previous
-
-
 def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask_mode, scale, q_pos, k_pos, q_seq,
                              k_seq) -> None:
     _check_attn_inputs(q, k, v)
@@ -234,10 +217,6 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
         raise ValueError(f"attention_backward: {why.decode()}")
     plan = _attach_doc_plan(shape, given, (q_pos, k_pos, q_seq, k_seq), q.device)  # noqa: F841 (alive over the launch)
     ws_bytes = L.mlts_attn_bwd_workspace_bytes(C.byref(shape), int(accumulate))
-    if _BWD_DS_HANDOVER_MAX_BYTES > 0:
-        ds_bytes = L.mlts_attn_bwd_ds_handover_bytes(C.byref(shape), int(accumulate))
-        if 0 < ds_bytes <= _BWD_DS_HANDOVER_MAX_BYTES:
-            ws_bytes += ds_bytes
     ws = _workspace(ws_bytes, q.device)
     _lib.check(
         L.mlts_attn_bwd(C.byref(shape), _p(dout), strides3(dout.stride()[:3]), _p(q), _p(k), _p(v), _p(o), _p(lse),

@@ -158,19 +158,25 @@ def test_cfg3_packed_documents_gqa_bf16_full_size(dev):
     o, lse = ops.attention(qg, kg, vg, mask_mode=ops.MASK_DOC, return_lse=True, **ids)
     o.backward(do)
     work = 0
+    worst = dict(O=0.0, dQ=0.0, dK=0.0, dV=0.0, LSE=0.0)
     for b in range(B):
         for start, L in docs[b]:
             sl = slice(start, start + L)
             qf, kf, vf = (t[b:b + 1, :, sl].float().requires_grad_(True) for t in (q, k, v))
             want_o, want_lse = oa.attention_with_lse(qf, kf, vf, oa.causal_mask(L, L, dev))  # K/V head = h // 4
             want_o.backward(do[b:b + 1, :, sl].float())
-            check_bf16(o[b:b + 1, :, sl], want_o, f"O[{b},{start}]")
-            assert (lse[b:b + 1, :, sl] - want_lse).abs().max() <= 2e-3
-            check_bf16(qg.grad[b:b + 1, :, sl], qf.grad, f"dQ[{b},{start}]")
-            check_bf16(kg.grad[b:b + 1, :, sl], kf.grad, f"dK[{b},{start}]")  # summed over the 4-head group
-            check_bf16(vg.grad[b:b + 1, :, sl], vf.grad, f"dV[{b},{start}]")
+            worst["O"] = max(worst["O"], check_bf16(o[b:b + 1, :, sl], want_o, f"O[{b},{start}]"))
+            worst["LSE"] = max(worst["LSE"], (lse[b:b + 1, :, sl] - want_lse).abs().max().item())
+            worst["dQ"] = max(worst["dQ"], check_bf16(qg.grad[b:b + 1, :, sl], qf.grad, f"dQ[{b},{start}]"))
+            worst["dK"] = max(worst["dK"], check_bf16(kg.grad[b:b + 1, :, sl], kf.grad, f"dK[{b},{start}]"))  # summed over the 4-head group
+            worst["dV"] = max(worst["dV"], check_bf16(vg.grad[b:b + 1, :, sl], vf.grad, f"dV[{b},{start}]"))
             work += L * L // 2
-    print(f"cfg3 documents per row: {[len(d) for d in docs]}, score elements/head: {work}")
+    print(f"cfg3 documents per row: {[len(d) for d in docs]}, score elements/head: {work}; max abs errors: {worst}")
+    assert worst["LSE"] <= 2e-3
+    # the stated bar without the half-ulp allowance.  dK and dV are sums over the four query heads of a KV head, so
+    # their values (and the half ulp of their rounding) are twice as large as with one head per KV head
+    for name in ("O", "dQ"):
+        assert worst[name] <= 2e-2, f"{name}: max abs error {worst[name]:.4f} above 2e-2"
 
 
 # ------------------------------------------------------------------ cfg4
@@ -189,17 +195,22 @@ def test_cfg4_zigzag_ring_rank_share_bf16_full_size(dev, rank):
     do_masked = torch.zeros_like(gdo)
     do_masked[:, :, pos[rank]] = gdo[:, :, pos[rank]]
     mask = oa.causal_mask(total, total, dev)
+    worst = dict(O=0.0, dQ=0.0, dK=0.0, dV=0.0, LSE=0.0)
     for h in range(H):
         qf, kf, vf = (t[:, h:h + 1].float().requires_grad_(True) for t in (gq, gk, gv))
         want_o, want_lse = oa.attention_with_lse(qf, kf, vf, mask)
         want_o.backward(do_masked[:, h:h + 1].float())
-        check_bf16(out[:, h:h + 1], want_o.detach()[:, :, pos[rank]], f"O head {h}")
-        assert (lse[:, h:h + 1] - want_lse.detach()[:, :, pos[rank]]).abs().max() <= 2e-3
-        check_bf16(q.grad[:, h:h + 1], qf.grad[:, :, pos[rank]], f"dQ head {h}")
+        worst["O"] = max(worst["O"], check_bf16(out[:, h:h + 1], want_o.detach()[:, :, pos[rank]], f"O head {h}"))
+        worst["LSE"] = max(worst["LSE"], (lse[:, h:h + 1] - want_lse.detach()[:, :, pos[rank]]).abs().max().item())
+        worst["dQ"] = max(worst["dQ"], check_bf16(q.grad[:, h:h + 1], qf.grad[:, :, pos[rank]], f"dQ head {h}"))
         for src, (kc, vc) in enumerate(chunks):
-            check_bf16(kc.grad[:, h:h + 1], kf.grad[:, :, pos[src]], f"dK head {h} chunk {src}")
-            check_bf16(vc.grad[:, h:h + 1], vf.grad[:, :, pos[src]], f"dV head {h} chunk {src}")
+            worst["dK"] = max(worst["dK"], check_bf16(kc.grad[:, h:h + 1], kf.grad[:, :, pos[src]], f"dK head {h} chunk {src}"))
+            worst["dV"] = max(worst["dV"], check_bf16(vc.grad[:, h:h + 1], vf.grad[:, :, pos[src]], f"dV head {h} chunk {src}"))
         del qf, kf, vf, want_o, want_lse
+    print(f"cfg4 rank {rank} max abs errors: {worst}")
+    assert worst["LSE"] <= 2e-3
+    for name in ("O", "dQ", "dK", "dV"):  # the stated bar without the half-ulp allowance
+        assert worst[name] <= 2e-2, f"{name}: max abs error {worst[name]:.4f} above 2e-2"
 
 
 # ------------------------------------------------------------------ cfg5

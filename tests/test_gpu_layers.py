@@ -338,19 +338,3 @@ def test_grad_to_f32_and_norm(dev, n, src_dtype):
     assert abs(ops.sq_norm(dst).item() - 4 * want) <= 1e-12 * 4 * want
     ops.scale_(dst, 0.5)
     assert torch.equal(dst.cpu(), src.float())
-
-
-def test_matrix_rate_probe_runs_and_counts_its_flops(dev):
-    """The measurement aid behind bench.py's box_matrix_rate: runs, leaves finite sums, and its flop count is the launch's."""
-    import ctypes as C
-    from maltos_amd import _lib
-    L = _lib.lib()
-    blocks, iters = 64, 10
-    assert L.mlts_mfma_probe_flops(blocks, iters) == blocks * 8 * iters * 16 * 2 * 32 * 32 * 16
-    operands = torch.randn(32768).bfloat16().to(dev)
-    out = torch.full((blocks * 512,), float("nan"), device=dev)
-    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    _lib.check(L.mlts_mfma_probe(operands.data_ptr(), operands.numel(), out.data_ptr(), blocks, iters, stream))
-    torch.cuda.synchronize()
-    assert torch.isfinite(out).all() and out.abs().sum() > 0
-    assert L.mlts_mfma_probe(operands.data_ptr(), 100, out.data_ptr(), blocks, iters, stream) != 0  # too few operands

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(str(_lib.LIB_PATH))
     for name in names:
         assert hasattr(handle, name), f"{name} not exported by {_lib.LIB_PATH.name}"
-    assert _lib.lib().mlts_abi_version() == 3
+    assert _lib.lib().mlts_abi_version() == 4
 
 
 def test_entry_points_validate_before_launch():
@@ -59,14 +59,11 @@ def test_entry_points_validate_before_launch():
     assert L.mlts_attn_supports(ctypes.byref(shape)) is None
     assert L.mlts_attn_fwd_workspace_bytes(ctypes.byref(shape)) == 0
     assert L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 0) >= L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 1) > 0
-    # the workspace is O(B * Hq * Sq); the dS hand-over is a separate, optional amount (head_dim 128 only)
+    # the workspace is O(B * Hq * Sq)
     assert L.mlts_attn_bwd_workspace_bytes(ctypes.byref(shape), 0) < 64 * 1024
-    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 0) == 0
     shape.D = 128
     for arr in (shape.q_stride, shape.k_stride, shape.v_stride, shape.o_stride):
         arr[0], arr[1], arr[2] = 8 * 3 * 128, 128, 3 * 128
-    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 0) >= 2 * 1 * 3 * 8 * 8
-    assert L.mlts_attn_bwd_ds_handover_bytes(ctypes.byref(shape), 1) == 0
     # rows further apart than 2^24 elements are refused (the MFMA kernels address a tile's rows with 32-bit offsets)
     shape.k_stride[2] = 1 << 24
     assert b"2^24" in L.mlts_attn_supports(ctypes.byref(shape))
