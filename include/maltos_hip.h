@@ -129,8 +129,10 @@ int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_s
  * results as mlts_attn_bwd with a workspace of exactly mlts_attn_bwd_workspace_bytes (the recomputing backward); the
  * workspace is a buffer of MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE bytes inside the library image, one copy per GPU, held
  * until the process ends.  Shapes whose workspace is larger (about B * Hq * Sq > 1 M query rows; with MLTS_MASK_DOC
- * also B * Sq * Sk / 4 bytes of visibility bits, e.g. B * S * S beyond about 28 M) are rejected with MLTS_ERR_INVALID.  No hipMalloc / hipFree is made.  All calls on one GPU share that buffer: calls that may overlap
- * on one GPU (different streams, different threads) race; serialise them or use mlts_attn_bwd. */
+ * also B * Sq * Sk / 4 bytes of visibility bits, e.g. B * S * S beyond about 28 M) are rejected with MLTS_ERR_INVALID.  No hipMalloc / hipFree is made.  All calls on one GPU share that buffer.  Calls on
+ * different streams of one GPU are made to take turns (each waits for an event recorded behind the last), except calls
+ * recorded into a HIP graph: graphs that hold this call and may run at the same time on one GPU race on the buffer and
+ * must be ordered by the caller, or use mlts_attn_bwd with one workspace per graph. */
 #define MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE (8 << 20)
 int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
                           const void* k, const void* v, const void* o, const float* lse, void* dq,

@@ -76,9 +76,10 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, atten
             return ops.attention(q, k, v, mask_mode=ops.MASK_CAUSAL)
         if (q_sequence_ids is None) != (k_sequence_ids is None):
             raise ValueError("q_sequence_ids and k_sequence_ids must both be provided or both be None")
-        if q_sequence_ids is None:  # positions only: one document per row
-            q_sequence_ids = torch.zeros_like(q_positions)
-            k_sequence_ids = torch.zeros_like(k_positions)
+        if q_sequence_ids is None:  # positions only: one document per row (the zero ids are kept with the positions)
+            zero_ids = lambda pos: torch.zeros(pos.shape, dtype=torch.int32, device=pos.device)
+            q_sequence_ids = ops.derived_from(q_positions, "_maltos_hip_zero_ids", zero_ids)
+            k_sequence_ids = q_sequence_ids if k_positions is q_positions else ops.derived_from(k_positions, "_maltos_hip_zero_ids", zero_ids)
         return ops.attention(q, k, v, mask_mode=ops.MASK_DOC, q_pos=q_positions, k_pos=k_positions,
                              q_seq=q_sequence_ids, k_seq=k_sequence_ids)
 

@@ -43,6 +43,14 @@ const char* shape_problem(const mlts_attn_shape* s) {
       return "bf16 MFMA path needs strides that keep rows 16-byte aligned";
     if (s->q_stride[2] >= kMaxRowStride || s->k_stride[2] >= kMaxRowStride || s->v_stride[2] >= kMaxRowStride)
       return "bf16 MFMA path needs sequence strides below 2^24 elements";
+    if (s->mask_mode == MLTS_MASK_DOC) {
+      // the pre-pass launches one wavefront per (batch row, 64-query group, four 64-key tiles) and the kernels index the
+      // visibility words of a (group, tile) pair densely; both counts are kept in 32 bits (the plan of such a call would
+      // be B * Sq * Sk / 4 bytes = 2 TiB: far beyond the memory of one GPU)
+      const int64_t nq = (static_cast<int64_t>(s->Sq) + kAttnTile - 1) / kAttnTile, nk = (static_cast<int64_t>(s->Sk) + kAttnTile - 1) / kAttnTile;
+      if (static_cast<int64_t>(s->B) * nq * nk >= (int64_t{1} << 31))
+        return "MLTS_MASK_DOC: B * ceil(Sq/64) * ceil(Sk/64) must stay below 2^31 tile pairs";
+    }
   }
   return nullptr;
 }
@@ -236,9 +244,23 @@ constexpr int64_t kScratchBytes = MLTS_ATTN_BWD_NOALLOC_MAX_WORKSPACE;
 __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 void* g_scratch_addr[kMaxDevices] = {};
+// the last use of a device's scratch: an event behind the kernels of the last call and the stream they ran on.  A call
+// on another stream waits for that event first, so that calls on different streams of one GPU take turns.
+hipEvent_t g_scratch_event[kMaxDevices] = {};
+hipStream_t g_scratch_stream[kMaxDevices] = {};
+bool g_scratch_used[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-int scratch_for_current_device(void** out) {
+bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+int scratch_for_current_device(void** out, int* dev_out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -254,8 +276,13 @@ int scratch_for_current_device(void** out) {
       return MLTS_ERR_LAUNCH;
     }
     g_scratch_addr[dev] = ptr;
+    if (hipEventCreateWithFlags(&g_scratch_event[dev], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      g_scratch_event[dev] = nullptr;  // calls still work; calls on different streams are then the caller's to order
+    }
   }
   *out = g_scratch_addr[dev];
+  *dev_out = dev;
   return MLTS_OK;
 }
 
@@ -504,6 +531,7 @@ char* setup_stats(AttnParams& p, const mlts_attn_shape* s, bool backward, char* 
   p.doc_bits_k = a.bits_k;
   p.head_pack_shift = mlts_doc_head_pack_shift(s->Hq, s->Hkv);
   a.q_rows = 256 >> p.head_pack_shift;
+  // (B * nq * nk < 2^31 was checked with the shape, so these block counts and their sum fit 32 bits)
   a.n_chunks = static_cast<int>((nk + kDocBitsChunk - 1) / kDocBitsChunk);
   a.bits_blocks = static_cast<int>(B * nq * a.n_chunks);
   a.q_blocks = static_cast<int>(B * ((s->Sq + a.q_rows - 1) / a.q_rows));
@@ -617,10 +645,33 @@ extern "C" int mlts_attn_bwd_noalloc(const mlts_attn_shape* s, const void* dout,
                "(about B*Hq*Sq <= %lld query rows); use mlts_attn_bwd with a caller workspace",
                (long long)need, (long long)kScratchBytes, (long long)(kScratchBytes / 8 - 64));
   void* ws = nullptr;
-  int rc = scratch_for_current_device(&ws);
+  int dev = 0;
+  int rc = scratch_for_current_device(&ws, &dev);
   if (rc != MLTS_OK) return rc;
-  return attn_bwd_impl("mlts_attn_bwd_noalloc", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv,
-                       dv_stride, accumulate_f32, ws, need, static_cast<hipStream_t>(stream));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // Calls on different streams take turns on the scratch: this call waits for the event behind the last one.  Not
+  // while a stream is being captured (an event recorded outside the capture cannot be waited for inside it): graphs
+  // that hold this call and are replayed on different streams of one GPU must be ordered by the caller.
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  const bool ordered = g_scratch_event[dev] != nullptr && !stream_is_capturing(st);
+  if (ordered && g_scratch_used[dev] && g_scratch_stream[dev] != st) {
+    if (hipStreamWaitEvent(st, g_scratch_event[dev], 0) != hipSuccess) {
+      mlts_set_error("mlts_attn_bwd_noalloc: cannot order this call behind the last user of the scratch: %s",
+                     hipGetErrorString(hipGetLastError()));
+      return MLTS_ERR_LAUNCH;
+    }
+  }
+  rc = attn_bwd_impl("mlts_attn_bwd_noalloc", s, dout, do_stride, q, k, v, o, lse, dq, dq_stride, dk, dk_stride, dv,
+                     dv_stride, accumulate_f32, ws, need, st);
+  if (ordered) {
+    if (hipEventRecord(g_scratch_event[dev], st) == hipSuccess) {
+      g_scratch_stream[dev] = st;
+      g_scratch_used[dev] = true;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+  return rc;
 }
 
 extern "C" int mlts_attn_merge(float* out_acc, float* lse_acc, const void* o_blk, const int64_t o_blk_stride[3],

@@ -104,13 +104,19 @@ def flash_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sequenc
     across runs, zeros at padding.  Runs directly on the padded [B, H, S, D] tensors: no gather/scatter."""
     if sequence_ids.dim() != 2 or sequence_ids.shape != (q.size(0), q.size(2)):
         raise ValueError(f"sequence_ids shape must match q/k/v batch+seq dimensions, got {tuple(sequence_ids.shape)}")
-    ids = sequence_ids.to(q.device)
-    valid = ids != PAD_SEQUENCE_ID
-    left_valid = torch.roll(valid, 1, dims=1)
-    left_valid[:, 0] = False
-    starts = valid & (~left_valid | (ids != torch.roll(ids, 1, dims=1)))
-    run_ids = torch.where(valid, starts.long().cumsum(dim=1) - 1, torch.full_like(ids, PAD_SEQUENCE_ID))
-    index = torch.arange(ids.size(1), device=ids.device, dtype=torch.long).unsqueeze(0).expand_as(ids)
+    device = q.device
+
+    def run_ids_and_index(sequence_ids):  # int32, what the kernels take; formed once per id tensor, not once per layer
+        ids = sequence_ids.to(device)
+        valid = ids != PAD_SEQUENCE_ID
+        left_valid = torch.roll(valid, 1, dims=1)
+        left_valid[:, 0] = False
+        starts = valid & (~left_valid | (ids != torch.roll(ids, 1, dims=1)))
+        run_ids = torch.where(valid, starts.long().cumsum(dim=1) - 1, torch.full_like(ids, PAD_SEQUENCE_ID, dtype=torch.long))
+        index = torch.arange(ids.size(1), device=device, dtype=torch.int32).unsqueeze(0).expand_as(ids)
+        return run_ids.to(torch.int32), index.contiguous()
+
+    run_ids, index = ops.derived_from(sequence_ids, f"_maltos_hip_run_ids_{device}", run_ids_and_index)
     return ops.attention(q, k, v, mask_mode=ops.MASK_DOC, q_pos=index, k_pos=index, q_seq=run_ids, k_seq=run_ids)
 
 
@@ -221,7 +227,10 @@ def varlen_prefix_metadata(*, q_positions: torch.Tensor, k_positions: torch.Tens
 
 def _raise_on_empty_prefix(lse: torch.Tensor, q_sequence_ids: torch.Tensor) -> None:
     """`allow_empty_kv=False` of the reference (flash_utils.py:677-684) costs one device-to-host flag here: a valid
-    query whose LSE is -inf saw no key."""
+    query whose LSE is -inf saw no key.  The read stalls the stream, so it is left out while the stream is being
+    captured into a HIP graph (a replay could not raise anyway): such callers pass `allow_empty_kv=True`."""
+    if lse.is_cuda and torch.cuda.is_current_stream_capturing():
+        return
     unseen = torch.isinf(lse).all(dim=1) & (q_sequence_ids != PAD_SEQUENCE_ID)
     if bool(unseen.any()):
         b, s = (int(x) for x in torch.nonzero(unseen, as_tuple=False)[0])
@@ -259,7 +268,12 @@ def flash_attn_varlen_prefix_backward(dout: torch.Tensor, q: torch.Tensor, k: to
                                       metadata_cache_key: object | None = None
                                       ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dq, dk, dv) of one block from caller-supplied out / LSE, which may be a ring's merged ones (reference
-    :863-962).  Tokens outside every visible pair receive zeros, as the reference's scatter leaves them."""
+    :863-962).  Tokens outside every visible pair receive zeros, as the reference's scatter leaves them.
+
+    `allow_empty_kv=False` differs from the reference here: its packer raises from this block's metadata when a query
+    run has no key in THIS chunk; this function only sees the LSE it is handed and raises when that says a valid query
+    saw no key at all, which a merged LSE says only if no chunk held one.  The block's own forward
+    (`flash_attn_varlen_prefix_with_lse`), which every schedule runs first, makes the per-block check."""
     del metadata, metadata_cache, metadata_cache_key
     q_seq, k_seq = _prefix_ids(q, k, v, q_positions, k_positions, q_sequence_ids, k_sequence_ids)
     if not allow_empty_kv:

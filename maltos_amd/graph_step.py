@@ -67,6 +67,8 @@ class CapturedForwardBackward:
             loss.backward()
             return loss
 
+        from .optim import grad_write_listener, notify_grad_written
+        self._notify_grad_written = notify_grad_written
         # warm-up on a side stream (workspaces, lazily created module state, library handles), then record on the SAME
         # stream: autograd ties each parameter's gradient accumulator to the stream of the forward pass that created it
         side = torch.cuda.Stream()
@@ -78,8 +80,13 @@ class CapturedForwardBackward:
         torch.cuda.synchronize()
         self._check_grads_in_place()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, stream=side):
-            self.loss = forward_backward()
+        # the parameters whose gradient the recorded backward writes: reported again after every replay, for optimizers
+        # that skip parameters without a gradient (a replay runs no Python, so nobody else would tell them)
+        with grad_write_listener() as seen, torch.cuda.graph(self.graph, stream=side):
+            # detached: nobody differentiates through the static loss, and an autograd graph kept alive here would tie
+            # the parameters' gradient accumulators to the recording stream for later eager passes
+            self.loss = forward_backward().detach()
+        self._written = list({id(p): p for p in seen}.values())
         self._check_grads_in_place()
         clear()            # the warm-up passes ran for real; recording itself executes nothing
 
@@ -110,6 +117,8 @@ class CapturedForwardBackward:
                 dst.copy_(src, non_blocking=True)
         self._check_grads_in_place()
         self.graph.replay()
+        for p in self._written:
+            self._notify_grad_written(p)
         if hidden is not None and hidden.requires_grad:
             hidden.backward(self._hidden.grad)      # eager: the embedding's own gradient
         return self.loss

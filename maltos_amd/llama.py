@@ -21,6 +21,7 @@ from .attn_masking_utils import canonical_position_ids, canonical_sequence_ids
 from .constants import (HIDDEN_STATES_KEY, INPUT_IDS_KEY, LABELS_KEY, LOSS_WEIGHT_KEY, POSITION_IDS_KEY,
                         POSITION_OFFSET_KEY, SEQUENCE_IDS_KEY)
 from .losses import causal_cross_entropy
+from .optim import notify_grad_written
 
 
 @dataclass(frozen=True)
@@ -39,6 +40,10 @@ class LlamaConfig:
     # each residual add is done inside the RMSNorm kernel that follows it (same values; one pass less per sublayer,
     # forward and backward); False keeps the reference's op sequence
     fuse_residual_norm: bool = True
+    # when the model computes the loss itself, the loss kernel writes the logits' gradient over the logits (no second
+    # buffer of their size).  Nobody else may then read the lm_head output of that forward; the model falls back to a
+    # separate gradient buffer by itself while lm_head carries forward hooks (which see that output).  False: always separate
+    loss_overwrites_logits: bool = True
 
     def __post_init__(self) -> None:
         validate_attention_backend(self.attention_backend)
@@ -88,6 +93,8 @@ class _SplitKLinearFn(torch.autograd.Function):
                 grad.addmm_(dy2.t(), x2)
             else:
                 dw = dy2.t().matmul(x2)
+            if grad is not None:
+                notify_grad_written(weight)   # autograd's hooks on the weight do not fire for a gradient added here
         return dx, dw, None
 
 
@@ -276,6 +283,14 @@ class LlamaForCausalLM(nn.Module):
             raise ValueError("LlamaForCausalLM requires input_ids or hidden_states")
         else:
             x = self.embed_tokens(input_ids)
+        if position_ids is not None or sequence_ids is not None:
+            # canonical [batch, seq] ids once per forward: every layer's attention is then handed the SAME tensors and
+            # shares what is derived from them (int32 forms, the document-mask plan), where per-layer canonicalisation
+            # (models/llama.py:163-175 of the reference) makes fresh ones whenever the batch's ids are rank 1, not int64,
+            # on the host, or absent.  Positions made here carry position_offset, which the rotary kernel then ignores.
+            position_ids = canonical_position_ids(position_ids, batch_size=x.size(0), seq_len=x.size(1),
+                                                  position_offset=position_offset, device=x.device)
+            sequence_ids = canonical_sequence_ids(sequence_ids, batch_size=x.size(0), seq_len=x.size(1), device=x.device)
         if self.config.fuse_residual_norm and x.is_cuda and len(self.layers) > 0:
             pending = None
             for layer in self.layers:
@@ -292,7 +307,8 @@ class LlamaForCausalLM(nn.Module):
         if input_ids is not None and labels.shape != input_ids.shape:
             raise ValueError(f"labels shape must match input_ids shape, got {labels.shape} vs {input_ids.shape}")
         # the logits are this function's own and are not returned with the loss: their gradient may take their place
-        loss = causal_cross_entropy(logits, labels, overwrite_logits=logits.is_cuda and logits.is_contiguous())
+        own = self.config.loss_overwrites_logits and not self.lm_head._forward_hooks
+        loss = causal_cross_entropy(logits, labels, overwrite_logits=own and logits.is_cuda and logits.is_contiguous())
         return loss if loss_weight is None else loss * float(loss_weight)
 
     def context_parallel_spec(self) -> list[str]:

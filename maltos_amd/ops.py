@@ -73,12 +73,30 @@ def _dense_last(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 or t.size(-1) == 1 else t.contiguous()
 
 
+def derived_from(t: torch.Tensor, attr: str, build):
+    """`build(t)`, kept on the tensor object `t` until `t` is modified in place (its autograd version counter moves).
+    Every layer of a model is handed the same id tensors, so what is derived from them (their int32 form, run ids, a
+    zero id tensor) is formed once per batch instead of once per layer, and, being the same tensor objects in every
+    call, lets the calls share one document-mask plan.  Not kept for inference tensors (no version counter) nor under
+    HIP graph capture (a tensor allocated while capturing belongs to the graph's pool)."""
+    if t.is_inference() or (t.is_cuda and torch.cuda.is_current_stream_capturing()):
+        return build(t)
+    hit = t.__dict__.get(attr)
+    if hit is not None and hit[0] == t._version:
+        return hit[1]
+    value = build(t)
+    t.__dict__[attr] = (t._version, value)
+    return value
+
+
 def _ids32(t: torch.Tensor | None, batch: int, seq: int, what: str) -> torch.Tensor | None:
     if t is None:
         return None
     if t.shape != (batch, seq):
         raise ValueError(f"{what} must have shape ({batch}, {seq}), got {tuple(t.shape)}")
-    return t.to(dtype=torch.int32).contiguous()
+    if t.dtype == torch.int32 and t.is_contiguous():
+        return t
+    return derived_from(t, "_maltos_hip_int32", lambda x: x.to(dtype=torch.int32).contiguous())
 
 
 def _attn_shape(q, k, v, o, mask_mode, scale, q_pos, k_pos, q_seq, k_seq) -> AttnShape:

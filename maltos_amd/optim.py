@@ -26,6 +26,35 @@ import torch.nn as nn
 from . import ops
 
 
+# Which parameters received a gradient in this step.  With gradients bound to a flat buffer `param.grad` is never None,
+# so "no gradient" (which the reference's optimizers skip, runtime/optim.py:46-50) has to be told another way: whoever
+# writes a parameter's gradient says so.  Autograd's own accumulation says it through a post-accumulate-grad hook that
+# the flat optimizer layout registers; code that adds into `param.grad` itself (HipLinear.accumulate_into_grad, a
+# replayed HIP graph, a reduce-scatter into a shard's gradient) calls notify_grad_written.
+_GRAD_WRITE_LISTENERS: list[list] = []
+
+
+def notify_grad_written(param: torch.Tensor) -> None:
+    mark = param.__dict__.get("_maltos_hip_grad_written")
+    if mark is not None:
+        mark()
+    for seen in _GRAD_WRITE_LISTENERS:
+        seen.append(param)
+
+
+class grad_write_listener:
+    """`with grad_write_listener() as seen:` collects the parameters whose gradient is reported written inside the block
+    (what a recorder of a backward pass keeps, to report the same parameters again after every replay)."""
+
+    def __enter__(self) -> list:
+        self._seen: list = []
+        _GRAD_WRITE_LISTENERS.append(self._seen)
+        return self._seen
+
+    def __exit__(self, *exc) -> None:
+        _GRAD_WRITE_LISTENERS.remove(self._seen)
+
+
 def _is_flat_neighbour(prev: torch.Tensor, nxt: torch.Tensor) -> bool:
     return (prev.untyped_storage().data_ptr() == nxt.untyped_storage().data_ptr()
             and prev.data_ptr() + prev.numel() * prev.element_size() == nxt.data_ptr())
@@ -178,11 +207,13 @@ class FusedAdamW(torch.optim.Optimizer):
                          weight_decay=float(group["weight_decay"]), sq_norm=sq_norm, max_norm=max_norm)
             for seg in self._segments[gi]:
                 flat_g = seg.flat_grad()
-                if flat_g is not None:
+                # one launch over the whole segment needs one step count (the bias corrections are launch arguments);
+                # the counts differ once a parameter was skipped in an earlier step for want of a gradient
+                steps = {float(self.state[p]["step"]) for p in seg.params}
+                if flat_g is not None and len(steps) == 1:
                     for p in seg.params:
                         self.state[p]["step"] += 1
-                    step = int(self.state[seg.params[0]]["step"].item())
-                    ops.adamw_step_(seg.flat_p, flat_g, seg.exp_avg, seg.exp_avg_sq, step=step,
+                    ops.adamw_step_(seg.flat_p, flat_g, seg.exp_avg, seg.exp_avg_sq, step=int(steps.pop()) + 1,
                                     p_lowp=self._shadow.get(seg.flat_p.data_ptr()), **hyper)
                     continue
                 shadow = self._shadow.get(seg.flat_p.data_ptr())
@@ -258,6 +289,12 @@ class MasterWeightsOptimizer(torch.optim.Optimizer):
                 self._optimizer.set_lowp_shadow(self.flat_master, self.flat_model)
         self.grad_sq_norm: torch.Tensor | None = None  # device fp64 scalar, filled by copy_master_params(fuse_norm=True)
         del total
+        # flat layout: which parameters' gradients were written since the last zero_grad (see notify_grad_written)
+        self._grad_written = [False] * len(model_params)
+        if self._flat_model:
+            for i, p in enumerate(model_params):
+                p.__dict__["_maltos_hip_grad_written"] = lambda i=i: self._grad_written.__setitem__(i, True)
+                p.register_post_accumulate_grad_hook(notify_grad_written)
 
     # ---- helpers --------------------------------------------------------------------------
     def _bind_model_grads(self) -> None:
@@ -275,6 +312,16 @@ class MasterWeightsOptimizer(torch.optim.Optimizer):
 
     def model_param_for(self, param: nn.Parameter) -> nn.Parameter:
         return self._model_param_by_master_id.get(id(param), param)
+
+    def mark_grads_written(self, params: Iterable[nn.Parameter] | None = None) -> None:
+        """For code that fills the bound `.grad` views itself, without autograd: these parameters (default: all) have a
+        gradient this step.  Parameters nobody reported are skipped by `step()`, as parameters whose `.grad` is None
+        are by the reference (runtime/optim.py:46-50)."""
+        if params is None:
+            self._grad_written = [True] * len(self.model_params)
+            return
+        for p in params:
+            notify_grad_written(p)
 
     # ---- reference API ----------------------------------------------------------------------
     def copy_master_params(self, fuse_norm: bool = False) -> None:
@@ -314,8 +361,22 @@ class MasterWeightsOptimizer(torch.optim.Optimizer):
 
     def step(self, closure=None):
         self.copy_master_params()
-        loss = self._optimizer.step(closure)
-        fused_writeback = self._fused and self._flat_model and all(mp.grad is not None for mp in self.master_params)
+        partial = self._flat_model and self._grads_are_flat() and not all(self._grad_written)
+        if partial:
+            # parameters without a gradient this step are left alone (no weight decay, no moment decay, no step count),
+            # like parameters whose .grad is None in the reference; the others are then stepped one launch each
+            for mp, written in zip(self.master_params, self._grad_written):
+                if not written:
+                    mp.grad = None
+        try:
+            loss = self._optimizer.step(closure)
+        finally:
+            if partial:
+                for mp, off in zip(self.master_params, self._offsets):
+                    if mp.grad is None:
+                        mp.grad = self.flat_master_grad[off:off + mp.numel()].view_as(mp)
+        # the fused step has written the bf16 model copy of everything it stepped
+        fused_writeback = self._fused and self._flat_model and (partial or all(mp.grad is not None for mp in self.master_params))
         if not fused_writeback:
             with torch.no_grad():
                 for p, mp in zip(self.model_params, self.master_params):
@@ -328,6 +389,7 @@ class MasterWeightsOptimizer(torch.optim.Optimizer):
             assert self.flat_model_grad is not None
             self.flat_model_grad.zero_()
             self._bind_model_grads()
+            self._grad_written = [False] * len(self.model_params)
         else:
             for p in self.model_params:
                 if set_to_none:

@@ -150,6 +150,11 @@ class Zero1FlatBuffers:
                 bucket.local_param.grad.copy_(full_grad[bucket.shard_start - bucket.start:bucket.shard_end - bucket.start])
             else:
                 self._reduce_scatter_avg(bucket.local_param.grad, full_grad)
+        # the shards' gradients were filled by hand, not by autograd: tell an optimizer that skips parameters without a
+        # gradient that every shard has one (the reference's ZeRO plugins step every shard, zero1.py:214-234)
+        mark = getattr(self.optimizer, "mark_grads_written", None)
+        if callable(mark):
+            mark()
 
     # ---- PRE_STEP: zero_common.py:307-351, zero1.py:214-234 ---------------------------------------------------
     def local_sq_norm(self) -> torch.Tensor:

@@ -207,6 +207,55 @@ def test_document_plan_is_reused_and_follows_the_ids(dev, D):
     check(o2, want, torch.bfloat16, "O after the ids changed in place")
 
 
+@pytest.mark.parametrize("ids_form", ["sequence-ids-only", "rank1-int32-host-positions"])
+def test_model_step_builds_one_document_plan_for_all_layers(dev, ids_form):
+    """A three-layer model step whose batch carries document ids runs the document-mask pre-pass ONCE (counted through
+    the library's timer on it): the model canonicalises the ids once per forward, so all layers, forward and backward,
+    hand the attention the same tensors; also through flash_attn_varlen, whose run ids are kept with the id tensor."""
+    from maltos_amd import _lib
+    from maltos_amd.constants import INPUT_IDS_KEY, LABELS_KEY, POSITION_IDS_KEY, SEQUENCE_IDS_KEY
+    from maltos_amd.flash_utils import flash_attn_varlen
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+
+    B, S = 2, 200
+    gen = torch.Generator().manual_seed(77)
+    cfg = LlamaConfig(vocab_size=512, hidden_size=256, intermediate_size=344, num_hidden_layers=3, num_attention_heads=4,
+                      num_key_value_heads=2, max_position_embeddings=S)
+    torch.manual_seed(5)
+    model = LlamaForCausalLM(cfg).to(dev).to(torch.bfloat16)
+    ids = torch.randint(0, 512, (B, S + 1), generator=gen)
+    pos, seq = make_docs(B, S, gen, 60, pad_tail=0)
+    batch = {INPUT_IDS_KEY: ids[:, :-1].to(dev), LABELS_KEY: ids[:, 1:].to(dev), SEQUENCE_IDS_KEY: seq.to(dev)}
+    if ids_form == "rank1-int32-host-positions":   # ids that the per-layer canonicalisation would copy afresh per layer
+        batch[POSITION_IDS_KEY] = torch.arange(S, dtype=torch.int32)
+        batch[SEQUENCE_IDS_KEY] = seq.int()
+    ops.clear_doc_plan_cache()
+    _lib.kernel_timing(True)
+    try:
+        model(batch).backward()
+        torch.cuda.synchronize()
+        _, builds = _lib.kernel_time_ms("attn_doc_prepass")
+    finally:
+        _lib.kernel_timing(False)
+    assert builds == 1, f"{builds} plan builds for 3 layers x (forward + backward)"
+    # the varlen provider function: three calls on one id tensor share the run ids and so the plan
+    q, k, v = (bshd(B, 2, S, 64, gen, torch.bfloat16).to(dev) for _ in range(3))
+    dseq = seq.to(dev)
+    ops.clear_doc_plan_cache()
+    _lib.kernel_timing(True)
+    try:
+        outs = [flash_attn_varlen(q, k, v, dseq) for _ in range(3)]
+        torch.cuda.synchronize()
+        _, builds = _lib.kernel_time_ms("attn_doc_prepass")
+    finally:
+        _lib.kernel_timing(False)
+    assert builds == 1 and torch.equal(outs[0], outs[2])
+    dseq[:, S // 2:] += 1   # edited in place: the kept run ids are not used any more
+    want, _ = oa.attention_with_lse(q.float().cpu(), k.float().cpu(), v.float().cpu(),
+                                    oa.doc_mask(*(2 * [torch.arange(S).repeat(B, 1)]), dseq.cpu(), dseq.cpu()))
+    check(flash_attn_varlen(q, k, v, dseq), want, torch.bfloat16, "varlen after the ids changed in place")
+
+
 @pytest.mark.parametrize("D", [1, 3, 24, 96, 192])
 def test_generic_head_dims(dev, D):
     run_case(dev, torch.float32, 1, 2, 1, 70, 70, D, ops.MASK_CAUSAL, seed=D)

@@ -338,3 +338,30 @@ def test_grad_to_f32_and_norm(dev, n, src_dtype):
     assert abs(ops.sq_norm(dst).item() - 4 * want) <= 1e-12 * 4 * want
     ops.scale_(dst, 0.5)
     assert torch.equal(dst.cpu(), src.float())
+
+
+def test_model_keeps_hooked_logits(dev):
+    """LlamaForCausalLM lets its loss write the gradient over the logits it owns; while lm_head carries a forward hook
+    (somebody sees that output), or with LlamaConfig.loss_overwrites_logits=False, the logits are left as they were.  The
+    loss and the gradients are the same in every form."""
+    from maltos_amd.llama import LlamaConfig, LlamaForCausalLM
+
+    gen = torch.Generator().manual_seed(11)
+    ids = torch.randint(0, 300, (2, 65), generator=gen).to(dev)
+    batch = (ids[:, :-1].contiguous(), ids[:, 1:].contiguous())
+    results = {}
+    for form in ("own", "hooked", "config-off"):
+        cfg = LlamaConfig(vocab_size=300, hidden_size=128, intermediate_size=256, num_hidden_layers=1, num_attention_heads=2,
+                          max_position_embeddings=64, loss_overwrites_logits=form != "config-off")
+        torch.manual_seed(3)
+        model = LlamaForCausalLM(cfg).to(dev).to(torch.bfloat16)
+        seen = []
+        if form != "own":
+            model.lm_head.register_forward_hook(lambda mod, args, out: seen.append((out, out.detach().clone())))
+        loss = model(batch)
+        loss.backward()
+        for out, copy in seen:
+            assert torch.equal(out.detach(), copy), f"{form}: the hooked logits were overwritten"
+        results[form] = (loss.detach().clone(), model.lm_head.weight.grad.clone())
+    for form in ("hooked", "config-off"):
+        assert torch.equal(results[form][0], results["own"][0]) and torch.equal(results[form][1], results["own"][1])

@@ -244,11 +244,11 @@ def test_linear_accumulates_weight_grad_into_bound_buffer(dev, rows, out_f, in_f
     assert fused.weight.grad is not None and (fused.weight.grad.double() - (exact - start.double())).abs().max() < 0.5
 
 
-def test_unused_parameter_is_skipped_in_the_per_parameter_layout(dev):
+def test_unused_parameter_is_skipped(dev):
     """A parameter that received no gradient: the reference leaves its master gradient at None and the inner optimizer
-    skips it (runtime/optim.py:46-50).  MasterWeightsOptimizer(flat=False) does the same; the flat layout (the default)
-    binds every gradient to a zeroed buffer, so there the parameter is stepped with a zero gradient (weight decay and
-    moment decay still apply) -- the documented difference."""
+    skips it (runtime/optim.py:46-50).  MasterWeightsOptimizer does the same in both layouts: per parameter
+    (flat=False) through `.grad is None`, flat (the default, every gradient bound to a buffer) through the record of
+    whose gradient was written this step."""
     used = nn.Parameter(torch.randn(8, 16, device=dev).bfloat16())
     unused = nn.Parameter(torch.randn(4, 16, device=dev).bfloat16())
     shadow = [used.detach().float().clone().requires_grad_(True), unused.detach().float().clone().requires_grad_(True)]
@@ -266,11 +266,34 @@ def test_unused_parameter_is_skipped_in_the_per_parameter_layout(dev):
     assert torch.equal(unused.detach(), before)                      # never touched, like the library's
     torch.testing.assert_close(opt.master_params[0].detach(), shadow[0].detach(), rtol=1e-4, atol=1e-7)
     torch.testing.assert_close(opt.master_params[1].detach(), shadow[1].detach(), rtol=0, atol=0)
-    # the flat layout steps it with a zero gradient: only the decoupled weight decay moves it
-    used2 = nn.Parameter(used.detach().clone())
-    unused2 = nn.Parameter(before.clone())
-    flat = MasterWeightsOptimizer([used2, unused2], optimizer_factory=lambda ps: FusedAdamW(ps, **HP), flat=True)
-    (used2.float() ** 2).sum().backward()
+    # the flat layout (the default): the same against the library, over steps in which the second parameter is unused,
+    # then used, then unused again (its step count and moments must follow the library's)
+    torch.manual_seed(4)
+    a = nn.Parameter(torch.randn(8, 16, device=dev).bfloat16())
+    b = nn.Parameter(torch.randn(4, 16, device=dev).bfloat16())
+    shadow = [a.detach().float().clone().requires_grad_(True), b.detach().float().clone().requires_grad_(True)]
+    lib = torch.optim.AdamW(shadow, **HP)
+    flat = MasterWeightsOptimizer([a, b], optimizer_factory=lambda ps: FusedAdamW(ps, **HP), flat=True)
+    assert flat.flat_model_grad is not None
+    for step, use_b in enumerate((False, True, False, False, True)):
+        loss = (a.float() ** 2).sum() + ((b.float() * 3).sin().sum() if use_b else 0.0)
+        loss.backward()
+        shadow[0].grad = a.grad.detach().float().clone()
+        shadow[1].grad = b.grad.detach().float().clone() if use_b else None
+        b_before = flat.master_params[1].detach().clone()
+        flat.step()
+        lib.step()
+        flat.zero_grad(set_to_none=True)
+        lib.zero_grad(set_to_none=True)
+        if not use_b:
+            assert torch.equal(flat.master_params[1].detach(), b_before), f"step {step}: the unused parameter moved"
+        for mp, sp, p_ in zip(flat.master_params, shadow, (a, b)):
+            torch.testing.assert_close(mp.detach(), sp.detach(), rtol=1e-4, atol=1e-7)
+            assert torch.equal(p_.detach(), mp.detach().to(torch.bfloat16))
+    assert float(flat.state[flat.master_params[1]]["step"]) == 2.0 and float(flat.state[flat.master_params[0]]["step"]) == 5.0
+    # gradients written by hand into the bound views are reported by hand
+    b.grad.fill_(0.5)
+    flat.mark_grads_written([b])
+    b_before = flat.master_params[1].detach().clone()
     flat.step()
-    want = before.float() * (1 - HP["lr"] * HP["weight_decay"])
-    torch.testing.assert_close(flat.master_params[1].detach(), want, rtol=1e-6, atol=1e-8)
+    assert not torch.equal(flat.master_params[1].detach(), b_before)

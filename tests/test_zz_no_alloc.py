@@ -63,6 +63,35 @@ def test_noalloc_backward_equals_workspace_backward_twice(dev, mode):
             assert torch.equal(a, b), f"{name} S={S}: no-alloc result differs from the workspace result"
 
 
+def test_noalloc_calls_on_two_streams_take_turns(dev):
+    """Two calls enqueued back to back on different streams share the one buffer: the second waits for the first (an
+    event behind the first call's kernels), so both give the results of the workspace form."""
+    L = _lib.lib()
+    mode = ops.MASK_CAUSAL
+    cases = [_inputs(dev, 2, 8, 8, 1500, 128, 21, mode), _inputs(dev, 1, 4, 4, 900, 128, 22, mode)]
+    want = []
+    for q, k, v, do, o, lse, kw in cases:
+        want.append(ops.attention_backward(do, q, k, v, o, lse, mask_mode=mode))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = []
+    p = lambda t: C.c_void_p(t.data_ptr())
+    for rep in range(3):
+        got.clear()
+        for (q, k, v, do, o, lse, kw), st in zip(cases, streams):
+            shape = ops._attn_shape(q, k, v, o, mode, q.size(-1) ** -0.5, None, None, None, None)
+            dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
+            st.wait_stream(torch.cuda.current_stream())
+            _lib.check(L.mlts_attn_bwd_noalloc(C.byref(shape), p(do), strides3(do.stride()[:3]), p(q), p(k), p(v), p(o), p(lse),
+                                               p(dq), strides3(dq.stride()[:3]), p(dk), strides3(dk.stride()[:3]), p(dv),
+                                               strides3(dv.stride()[:3]), 0, C.c_void_p(st.cuda_stream)))
+            got.append((dq, dk, dv))
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            for a, b in zip(g, w):
+                assert torch.equal(a, b), f"repetition {rep}: a call on its own stream differs from the workspace form"
+
+
 def test_noalloc_rejects_shapes_beyond_its_buffer(dev):
     """B * Hq * Sq rows whose statistics do not fit the built-in buffer are refused before any launch."""
     L = _lib.lib()
