@@ -115,9 +115,19 @@ int mlts_attn_fwd(const mlts_attn_shape* s, const void* q, const void* k, const 
 /* dQ, dK, dV by recompute from (Q, K, V, O, LSE, dO); O and LSE may be the GLOBAL ones of a ring
  * schedule, which is what makes per-block calls compose.  Replaces flash_attn_dense_backward
  * (runtime/layers/flash_utils.py:218-263) and the autograd of SDPA.
- * accumulate_f32 = 0: dq/dk/dv have the input dtype and are overwritten (strides dq_stride etc).
- * accumulate_f32 = 1: dq/dk/dv are fp32 and are ADDED to (the `dq += block_dq.float()` form of
- *                     runtime/layers/functional.py:1121-1146). */
+ * accumulate_f32 (strides dq_stride etc are in elements of the respective type):
+ *   MLTS_BWD_OVERWRITE (0)     dq/dk/dv have the input dtype and are overwritten.
+ *   MLTS_BWD_ACCUMULATE (1)    dq/dk/dv are fp32 and are ADDED to (the `dq += block_dq.float()` form of
+ *                              runtime/layers/functional.py:1121-1146).
+ *   MLTS_BWD_DQ_ACCUMULATE (2) dq is fp32 and added to; dk/dv have the input dtype and are overwritten: a block of a
+ *                              ring step on the rank that owns the queries, where a K/V chunk meets the local queries
+ *                              exactly once (functional.py:1104-1146: one `dk += ...` per chunk and rank).
+ *   MLTS_BWD_DQ_STORE (3)      as 2, but dq (fp32) is overwritten: the first block of such an accumulation, which
+ *                              saves clearing the fp32 buffer beforehand. */
+#define MLTS_BWD_OVERWRITE 0
+#define MLTS_BWD_ACCUMULATE 1
+#define MLTS_BWD_DQ_ACCUMULATE 2
+#define MLTS_BWD_DQ_STORE 3
 int mlts_attn_bwd(const mlts_attn_shape* s, const void* dout, const int64_t do_stride[3], const void* q,
                   const void* k, const void* v, const void* o, const float* lse, void* dq,
                   const int64_t dq_stride[3], void* dk, const int64_t dk_stride[3], void* dv,

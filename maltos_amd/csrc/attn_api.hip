@@ -193,6 +193,10 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
                   void* workspace, int64_t workspace_bytes, hipStream_t st) {
   MLTS_REQUIRE(dout && q && k && v && o && lse && dq && dk && dv, "%s: null tensor pointer", who);
   MLTS_REQUIRE(do_stride && dq_stride && dk_stride && dv_stride, "%s: null stride pointer", who);
+  MLTS_REQUIRE(accumulate_f32 >= MLTS_BWD_OVERWRITE && accumulate_f32 <= MLTS_BWD_DQ_STORE, "%s: unknown accumulate_f32 mode %d", who,
+               accumulate_f32);
+  const int dq_f32 = accumulate_f32 == MLTS_BWD_OVERWRITE ? 0 : accumulate_f32 == MLTS_BWD_DQ_STORE ? 2 : 1;
+  const int dkv_f32 = accumulate_f32 == MLTS_BWD_ACCUMULATE ? 1 : 0;
   const int64_t need = bwd_min_workspace(s);
   MLTS_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace too small (%lld < %lld)", who,
                (long long)workspace_bytes, (long long)need);
@@ -212,16 +216,16 @@ int attn_bwd_impl(const char* who, const mlts_attn_shape* s, const void* dout, c
     bp.dks[i] = dk_stride[i];
     bp.dvs[i] = dv_stride[i];
   }
-  bp.accumulate_f32 = accumulate_f32 ? 1 : 0;
+  bp.accumulate_f32 = dkv_f32;
+  bp.dq_f32 = dq_f32;
   bp.nkt = 0;
   bp.delta_out = bp.lse2_out = nullptr;
   if (uses_mfma(s)) {
     MLTS_REQUIRE(mlts_aligned16(dout) && mlts_aligned16(q) && mlts_aligned16(k) && mlts_aligned16(v) &&
                      mlts_aligned16(dq) && mlts_aligned16(dk) && mlts_aligned16(dv),
                  "%s: tensors must be 16-byte aligned", who);
-    const int es_out = accumulate_f32 ? 4 : 2;
-    MLTS_REQUIRE(strides_aligned(do_stride, 2) && strides_aligned(dq_stride, es_out) &&
-                     strides_aligned(dk_stride, es_out) && strides_aligned(dv_stride, es_out),
+    MLTS_REQUIRE(strides_aligned(do_stride, 2) && strides_aligned(dq_stride, dq_f32 ? 4 : 2) &&
+                     strides_aligned(dk_stride, dkv_f32 ? 4 : 2) && strides_aligned(dv_stride, dkv_f32 ? 4 : 2),
                  "%s: strides must keep rows 16-byte aligned", who);
     MLTS_REQUIRE(do_stride[2] < kMaxRowStride, "%s: the sequence stride of dout must be below 2^24 elements", who);
   }

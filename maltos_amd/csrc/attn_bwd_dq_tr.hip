@@ -519,7 +519,7 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
 
   const float oscale = -p.scale;  // the accumulator holds K^T (-dS^T)
   const bool rows16 = ((bp.dqs[0] | bp.dqs[1] | bp.dqs[2]) & 7) == 0 && (reinterpret_cast<uintptr_t>(bp.dq_acc) & 15) == 0;
-  if (!bp.accumulate_f32 && rows16) {
+  if (!bp.dq_f32 && rows16) {
     // bf16 rows through LDS (each wavefront owns 32 rows x RB bytes, tile-row swizzle), so that global stores are
     // 16 bytes per lane and cover whole rows
     drain_and_barrier();  // every wavefront has finished reading the last K/V tile
@@ -542,15 +542,15 @@ __global__ __launch_bounds__(THREADS) void attn_bwd_dq_tr_kernel(const AttnBwdPa
       const v4i32 x = *reinterpret_cast<const v4i32*>(ebase + row * RB + ((chunk ^ swz<D>(row & 15)) << 4));
       if (wq0 + row < p.Sq) *reinterpret_cast<v4i32*>(obase + static_cast<int64_t>(wq0 + row) * bp.dqs[2] + chunk * 8) = x;
     }
-  } else if (qrow < p.Sq && bp.accumulate_f32) {
+  } else if (qrow < p.Sq && bp.dq_f32) {
     // fp32 gradients that are added to (ring steps): all loads of the old values before the first store, one memory
-    // round trip instead of sixteen dependent ones
+    // round trip instead of sixteen dependent ones; the first block of an accumulation (dq_f32 == 2) stores only
     f32x4* dst = reinterpret_cast<f32x4*>(bp.dq_acc + b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(qrow) * bp.dqs[2] + hh * 4);
     f32x4 cur[DB][4];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) cur[db][g] = dst[db * 8 + g * 2];
+      for (int g = 0; g < 4; ++g) cur[db][g] = bp.dq_f32 == 2 ? f32x4{0.f, 0.f, 0.f, 0.f} : dst[db * 8 + g * 2];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll

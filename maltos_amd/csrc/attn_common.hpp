@@ -56,12 +56,13 @@ struct AttnBwdParams {
   const void* dout;
   int64_t dos[3];
   const float* delta;  // [B, Hq, Sq] rowsum(dO * O)
-  float* dq_acc;       // fp32 [B, Hq, Sq, D] accumulated with atomics (contiguous or caller strides)
+  float* dq_acc;       // dQ [B, Hq, Sq, D] with caller strides: the input dtype, or fp32 (dq_f32 != 0)
   int64_t dqs[3];
   void* dk;
   void* dv;
   int64_t dks[3], dvs[3];
-  int accumulate_f32;  // dk/dv are fp32 and added to
+  int accumulate_f32;  // dk/dv are fp32 and added to (otherwise the input dtype, overwritten)
+  int dq_f32;          // 0: dq has the input dtype and is overwritten; 1: fp32, added to; 2: fp32, overwritten
   int nkt;             // key tiles per (batch, kv head)
   // Optional outputs of the recomputing dQ kernel, which then runs first and takes the place of the separate row
   // statistics passes: delta_out[B, Hq, Sq] = rowsum(dO * O) (the kernel ignores `delta` and reads `a.o`), and

@@ -123,8 +123,8 @@ __global__ __launch_bounds__(GT) void attn_generic_fwd(const AttnParams p, int D
 }
 
 // dQ for 16 query rows: dq = scale * sum_j ds_ij k_j, ds = p (dp - delta), p = exp(scale s - lse).
-// DQ_F32_ACC: dq is fp32 and added to.
-template <typename T, int MODE, bool DQ_F32_ACC>
+// bp.dq_f32: dq is fp32 and added to (1) or overwritten (2); 0: dq has the input dtype.
+template <typename T, int MODE>
 __global__ __launch_bounds__(GT) void attn_generic_bwd_dq(const AttnBwdParams bp, int D) {
   const AttnParams& p = bp.a;
   extern __shared__ float lds[];
@@ -197,7 +197,8 @@ __global__ __launch_bounds__(GT) void attn_generic_bwd_dq(const AttnBwdParams bp
       const int d = lane + 64 * dd;
       if (d >= D) continue;
       const int64_t off = b * bp.dqs[0] + hq * bp.dqs[1] + static_cast<int64_t>(row) * bp.dqs[2] + d;
-      if (DQ_F32_ACC) bp.dq_acc[off] += dq[r][dd] * p.scale;
+      if (bp.dq_f32 == 1) bp.dq_acc[off] += dq[r][dd] * p.scale;
+      else if (bp.dq_f32 == 2) bp.dq_acc[off] = dq[r][dd] * p.scale;
       else reinterpret_cast<T*>(bp.dq_acc)[off] = from_f32<T>(dq[r][dd] * p.scale);
     }
   }
@@ -388,19 +389,16 @@ int generic_bwd_t(const AttnBwdParams& bp, int D, hipStream_t st) {
   const size_t lds = generic_lds_floats(D) * sizeof(float);
   dim3 gq((p.Sq + GROWS - 1) / GROWS, p.B * p.Hq);
   dim3 gk((p.Sk + GROWS - 1) / GROWS, p.B * p.Hkv);
+  auto kq = attn_generic_bwd_dq<T, MODE>;
+  if (int rc = set_lds(kq, lds, "mlts_attn_bwd")) return rc;
+  hipLaunchKernelGGL(kq, gq, dim3(GT), lds, st, bp, D);
   if (bp.accumulate_f32) {
-    auto kq = attn_generic_bwd_dq<T, MODE, true>;
     auto kk = attn_generic_bwd_dkv<T, MODE, true>;
-    if (int rc = set_lds(kq, lds, "mlts_attn_bwd")) return rc;
     if (int rc = set_lds(kk, lds, "mlts_attn_bwd")) return rc;
-    hipLaunchKernelGGL(kq, gq, dim3(GT), lds, st, bp, D);
     hipLaunchKernelGGL(kk, gk, dim3(GT), lds, st, bp, D);
   } else {
-    auto kq = attn_generic_bwd_dq<T, MODE, false>;
     auto kk = attn_generic_bwd_dkv<T, MODE, false>;
-    if (int rc = set_lds(kq, lds, "mlts_attn_bwd")) return rc;
     if (int rc = set_lds(kk, lds, "mlts_attn_bwd")) return rc;
-    hipLaunchKernelGGL(kq, gq, dim3(GT), lds, st, bp, D);
     hipLaunchKernelGGL(kk, gk, dim3(GT), lds, st, bp, D);
   }
   return mlts_check_launch("mlts_attn_bwd");

@@ -16,9 +16,13 @@ import torch
 from . import _lib
 from ._lib import MASK_CAUSAL, MASK_DOC, MASK_NONE, MLTS_BF16, MLTS_F32, AttnShape, strides3
 
+# mlts_attn_bwd's accumulate_f32 modes (include/maltos_hip.h)
+BWD_OVERWRITE, BWD_ACCUMULATE, BWD_DQ_ACCUMULATE, BWD_DQ_STORE = 0, 1, 2, 3
+
 __all__ = [
     "MASK_NONE", "MASK_CAUSAL", "MASK_DOC",
-    "attention", "attention_forward", "attention_backward", "attention_backward_accumulate", "attention_merge_",
+    "attention", "attention_forward", "attention_backward", "attention_backward_accumulate",
+    "attention_backward_ring_block", "attention_merge_",
     "rms_norm", "rope", "rope_pair", "swiglu", "cross_entropy",
     "adamw_step_", "sq_norm", "scale_", "grad_to_f32_",
 ]
@@ -216,8 +220,10 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
     B, Hq, Sq, D = q.shape
     Sk = k.size(2)
     if B == 0 or Sq == 0 or Sk == 0:
-        if not accumulate:
-            dq.zero_(), dk.zero_(), dv.zero_()
+        if accumulate in (BWD_OVERWRITE, BWD_DQ_STORE):
+            dq.zero_()
+        if accumulate != BWD_ACCUMULATE:
+            dk.zero_(), dv.zero_()
         return
     if dout.shape != q.shape or o.shape != q.shape:
         raise ValueError("dout and out must have the shape of q")
@@ -250,7 +256,7 @@ def attention_backward(dout, q, k, v, o, lse, *, mask_mode: int, scale: float | 
     dq = _bshd_empty(q.size(0), q.size(1), q.size(2), q.size(3), q)
     dk = _bshd_empty(k.size(0), k.size(1), k.size(2), k.size(3), k)
     dv = _bshd_empty(v.size(0), v.size(1), v.size(2), v.size(3), v)
-    _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, False, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
+    _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, BWD_OVERWRITE, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
     return dq, dk, dv
 
 
@@ -261,7 +267,22 @@ def attention_backward_accumulate(dout, q, k, v, o, lse, dq, dk, dv, *, mask_mod
         if t.dtype != torch.float32 or t.shape != ref.shape or t.stride(-1) != 1:
             raise ValueError(f"{name} must be float32 with the shape of its input and a contiguous head_dim")
     q, k, v, o, dout = map(_dense_last, (q, k, v, o, dout))
-    _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, True, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
+    _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, BWD_ACCUMULATE, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
+
+
+def attention_backward_ring_block(dout, q, k, v, o, lse, dq, dk, dv, *, first: bool, mask_mode: int, scale: float | None = None,
+                                  q_pos=None, k_pos=None, q_seq=None, k_seq=None) -> None:
+    """One block of a ring schedule on the rank that owns the queries: dq (fp32) collects every block (`first`: this
+    block overwrites it, so nobody has to clear it; later blocks add), while dk and dv of the block's keys (input
+    dtype) are written once, since a K/V chunk meets the local queries in exactly one block."""
+    if dq.dtype != torch.float32 or dq.shape != q.shape or dq.stride(-1) != 1:
+        raise ValueError("dq must be float32 with the shape of q and a contiguous head_dim")
+    for name, t, ref in (("dk", dk, k), ("dv", dv, v)):
+        if t.dtype != ref.dtype or t.shape != ref.shape or t.stride(-1) != 1:
+            raise ValueError(f"{name} must have the dtype and shape of its input and a contiguous head_dim")
+    q, k, v, o, dout = map(_dense_last, (q, k, v, o, dout))
+    _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, BWD_DQ_STORE if first else BWD_DQ_ACCUMULATE, mask_mode, scale,
+                             q_pos, k_pos, q_seq, k_seq)
 
 
 def attention_merge_(out_acc, lse_acc, o_blk, lse_blk, q_off: int = 0) -> None:

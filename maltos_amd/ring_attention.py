@@ -46,16 +46,12 @@ def zigzag_ring_schedule(rank: int, world_size: int) -> list[tuple[int, str]]:
     return plan
 
 
-def _chunk_grad_buffers(ks, device):
-    """Zeroed fp32 dK, dV of every chunk: [2 * chunks, ...] in one buffer when the chunks have one shape (one fill and
-    one conversion instead of two per chunk), else a list."""
-    if all(k.shape == ks[0].shape for k in ks):
-        return torch.zeros((2 * len(ks), *ks[0].shape), dtype=torch.float32, device=device)
-    return [torch.zeros(k.shape, dtype=torch.float32, device=device) for k in ks for _ in range(2)]
-
-
-def _chunk_grads(dkv, dtype):
-    return dkv.to(dtype).unbind(0) if isinstance(dkv, torch.Tensor) else [g.to(dtype) for g in dkv]
+def _first_block_state(blk) -> tuple[torch.Tensor, torch.Tensor]:
+    """The running fp32 (out, lse) of a schedule whose first block covers every local query: that block itself (one
+    conversion instead of clearing the state and merging the block into it)."""
+    running_out = torch.empty(blk.out.shape, dtype=torch.float32, device=blk.out.device)
+    running_out.copy_(blk.out)
+    return running_out, blk.lse
 
 
 class _ZigzagRingFunction(torch.autograd.Function):
@@ -67,13 +63,11 @@ class _ZigzagRingFunction(torch.autograd.Function):
         if seq % 2:
             raise ValueError(f"zigzag ring attention requires an even local sequence length, got {seq}")
         half = seq // 2
-        running_out = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-        running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+        running_out = running_lse = None
         for src, kind in zigzag_ring_schedule(rank, world_size):
             k, v = kv_flat[2 * src], kv_flat[2 * src + 1]
-            if kind == "causal":
-                blk = flash_attn_dense_with_lse(q, k, v, causal=True)
-                ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, 0)
+            if kind == "causal":  # step 0, all local queries
+                running_out, running_lse = _first_block_state(flash_attn_dense_with_lse(q, k, v, causal=True))
             elif kind == "front_kv":
                 blk = flash_attn_dense_with_lse(q, k[:, :, :half], v[:, :, :half], causal=False)
                 ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, 0)
@@ -92,21 +86,35 @@ class _ZigzagRingFunction(torch.autograd.Function):
         rank, world_size = ctx.rank, ctx.world_size
         half = q.size(-2) // 2
         dout = dout.contiguous()
-        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-        dkv = _chunk_grad_buffers(kv_flat[0::2], q.device)
-        for src, kind in zigzag_ring_schedule(rank, world_size):
+        # dq collects every step in fp32: the first step (causal, all local queries) overwrites it, the others add.
+        # A chunk's dK / dV come from exactly one step, so that step writes them in their final dtype; only the half
+        # of a chunk that a front_kv step does not touch is cleared.
+        dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+        grads: list[torch.Tensor | None] = [None] * len(kv_flat)
+        for step, (src, kind) in enumerate(zigzag_ring_schedule(rank, world_size)):
             k, v = kv_flat[2 * src], kv_flat[2 * src + 1]
-            dk, dv = dkv[2 * src], dkv[2 * src + 1]
+            dk, dv = torch.empty_like(k), torch.empty_like(v)
+            grads[2 * src], grads[2 * src + 1] = dk, dv
             if kind == "causal":
-                ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dk, dv, mask_mode=ops.MASK_CAUSAL)
+                ops.attention_backward_ring_block(dout, q, k, v, out, lse, dq, dk, dv, first=step == 0, mask_mode=ops.MASK_CAUSAL)
             elif kind == "front_kv":
-                ops.attention_backward_accumulate(dout, q, k[:, :, :half], v[:, :, :half], out, lse, dq, dk[:, :, :half],
-                                                  dv[:, :, :half], mask_mode=ops.MASK_NONE)
+                dk[:, :, half:].zero_()
+                dv[:, :, half:].zero_()
+                ops.attention_backward_ring_block(dout, q, k[:, :, :half], v[:, :, :half], out, lse, dq, dk[:, :, :half],
+                                                  dv[:, :, :half], first=False, mask_mode=ops.MASK_NONE)
             else:
-                ops.attention_backward_accumulate(dout[:, :, half:], q[:, :, half:], k, v, out[:, :, half:],
-                                                  lse[:, :, half:].contiguous(), dq[:, :, half:], dk, dv,
+                ops.attention_backward_ring_block(dout[:, :, half:], q[:, :, half:], k, v, out[:, :, half:],
+                                                  lse[:, :, half:].contiguous(), dq[:, :, half:], dk, dv, first=False,
                                                   mask_mode=ops.MASK_NONE)
-        return (dq.to(q.dtype), None, None, *_chunk_grads(dkv, kv_flat[0].dtype))
+        return (dq.to(q.dtype), None, None, *grads)
+
+
+def flash_attn_dense_block(q, k, v, q_pos, k_pos, q_seq, k_seq):
+    """One document-masked block without autograd: (out, lse) as flash_attn_dense_with_lse returns them."""
+    from .flash_utils import FlashAttnBlockOutput
+
+    out, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, q_pos=q_pos, k_pos=k_pos, q_seq=q_seq, k_seq=k_seq)
+    return FlashAttnBlockOutput(out=out, lse=lse)
 
 
 class _PackedRingFunction(torch.autograd.Function):
@@ -116,13 +124,14 @@ class _PackedRingFunction(torch.autograd.Function):
     def forward(ctx, q: torch.Tensor, q_pos: torch.Tensor, q_seq: torch.Tensor, rank: int, world_size: int, *flat):
         if len(flat) != 4 * world_size:
             raise ValueError(f"expected {4 * world_size} chunk tensors, got {len(flat)}")
-        running_out = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-        running_lse = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+        running_out = running_lse = None
         for step in range(world_size):
             k, v, k_pos, k_seq = flat[4 * ((rank - step) % world_size):][:4]
-            o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_DOC, q_pos=q_pos, k_pos=k_pos, q_seq=q_seq,
-                                           k_seq=k_seq)
-            ops.attention_merge_(running_out, running_lse, o, lse, 0)  # a block nobody sees into is (0, -inf)
+            blk = flash_attn_dense_block(q, k, v, q_pos, k_pos, q_seq, k_seq)
+            if step == 0:
+                running_out, running_lse = _first_block_state(blk)
+            else:
+                ops.attention_merge_(running_out, running_lse, blk.out, blk.lse, 0)  # a block nobody sees into is (0, -inf)
         out = running_out.to(dtype=flat[1].dtype)
         ctx.save_for_backward(q, q_pos, q_seq, out, running_lse, *flat)
         ctx.rank, ctx.world_size = rank, world_size
@@ -134,17 +143,15 @@ class _PackedRingFunction(torch.autograd.Function):
         q, q_pos, q_seq, out, lse, *flat = ctx.saved_tensors
         rank, world_size = ctx.rank, ctx.world_size
         dout = dout.contiguous()
-        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)  # the first step overwrites it, the others add
         grads: list[torch.Tensor | None] = [None] * (4 * world_size)
-        dkv = _chunk_grad_buffers(flat[0::4], q.device)
         for step in range(world_size):
             src = (rank - step) % world_size
             k, v, k_pos, k_seq = flat[4 * src:][:4]
-            ops.attention_backward_accumulate(dout, q, k, v, out, lse, dq, dkv[2 * src], dkv[2 * src + 1], mask_mode=ops.MASK_DOC,
+            dk, dv = torch.empty_like(k), torch.empty_like(v)  # every step sees the whole chunk: written once, in place
+            grads[4 * src], grads[4 * src + 1] = dk, dv
+            ops.attention_backward_ring_block(dout, q, k, v, out, lse, dq, dk, dv, first=step == 0, mask_mode=ops.MASK_DOC,
                                               q_pos=q_pos, k_pos=k_pos, q_seq=q_seq, k_seq=k_seq)
-        dkv = _chunk_grads(dkv, flat[0].dtype)
-        for src in range(world_size):
-            grads[4 * src], grads[4 * src + 1] = dkv[2 * src], dkv[2 * src + 1]
         return (dq.to(q.dtype), None, None, None, None, *grads)
 
 

@@ -256,6 +256,43 @@ def test_model_step_builds_one_document_plan_for_all_layers(dev, ids_form):
     check(flash_attn_varlen(q, k, v, dseq), want, torch.bfloat16, "varlen after the ids changed in place")
 
 
+@pytest.mark.parametrize("dtype,D,mode", [(torch.bfloat16, 128, ops.MASK_CAUSAL), (torch.bfloat16, 64, ops.MASK_NONE),
+                                          (torch.bfloat16, 128, ops.MASK_DOC), (torch.float32, 24, ops.MASK_CAUSAL)])
+def test_backward_accumulation_modes(dev, dtype, D, mode):
+    """mlts_attn_bwd's output modes against the plain one (everything in the input dtype, overwritten): fp32 gradients
+    that are added to (all three, or dQ only with dK / dV written once in the input dtype) and the first block of such
+    an accumulation, which overwrites the fp32 dQ instead of adding to it."""
+    B, Hq, Hkv, Sq, Sk = 2, 4, 2, 333, 333
+    gen = torch.Generator().manual_seed(400 + D)
+    q, k, v, do = (bshd(B, h, s, D, gen, dtype).to(dev) for h, s in ((Hq, Sq), (Hkv, Sk), (Hkv, Sk), (Hq, Sq)))
+    kw = {}
+    if mode == ops.MASK_DOC:
+        pos, seq = make_docs(B, Sq, gen, 90, pad_tail=7)
+        kw = dict(q_pos=pos.to(dev), k_pos=pos.to(dev), q_seq=seq.to(dev), k_seq=seq.to(dev))
+    o, lse = ops.attention_forward(q, k, v, mask_mode=mode, **kw)
+    dq0, dk0, dv0 = ops.attention_backward(do, q, k, v, o, lse, mask_mode=mode, **kw)
+    nan32 = lambda t: torch.full(t.shape, float("nan"), dtype=torch.float32, device=dev)
+    # first block of an accumulation: dq (fp32) and dk, dv (input dtype) are all overwritten
+    dq, dk, dv = nan32(q), torch.full_like(k, float("nan")), torch.full_like(v, float("nan"))
+    ops.attention_backward_ring_block(do, q, k, v, o, lse, dq, dk, dv, first=True, mask_mode=mode, **kw)
+    assert torch.equal(dq.to(dtype), dq0) and torch.equal(dk, dk0) and torch.equal(dv, dv0)
+    # a later block: dq is added to, dk and dv are overwritten again
+    first = dq.clone()
+    dk.fill_(float("nan")), dv.fill_(float("nan"))
+    ops.attention_backward_ring_block(do, q, k, v, o, lse, dq, dk, dv, first=False, mask_mode=mode, **kw)
+    assert torch.equal(dq, first + first) and torch.equal(dk, dk0) and torch.equal(dv, dv0)
+    # everything in fp32, added to
+    dq, dk, dv = torch.ones_like(first), torch.ones(k.shape, device=dev), torch.ones(v.shape, device=dev)
+    ops.attention_backward_accumulate(do, q, k, v, o, lse, dq, dk, dv, mask_mode=mode, **kw)
+    tol = dict(rtol=1e-6, atol=1e-6)
+    assert torch.allclose(dq, first + 1, **tol)   # (the product and the addition may be one fused operation)
+    if dtype == torch.bfloat16:  # the fp32 values round to what the plain form stored
+        assert torch.equal((dk - 1).to(dtype), dk0) or torch.allclose((dk - 1), dk0.float(), rtol=2.0 ** -7, atol=1e-5)
+        assert torch.allclose(dv - 1, dv0.float(), rtol=2.0 ** -7, atol=1e-5)
+    else:
+        assert torch.allclose(dk - 1, dk0, **tol) and torch.allclose(dv - 1, dv0, **tol)
+
+
 @pytest.mark.parametrize("D", [1, 3, 24, 96, 192])
 def test_generic_head_dims(dev, D):
     run_case(dev, torch.float32, 1, 2, 1, 70, 70, D, ops.MASK_CAUSAL, seed=D)
