@@ -210,6 +210,14 @@ int mlts_swiglu_fwd(const void* gate, const void* up, void* h, int64_t n, int32_
 int mlts_swiglu_bwd(const void* dh, const void* gate, const void* up, void* dgate, void* dup, int64_t n,
                     int32_t dtype, mlts_stream_t stream);
 
+/* The same over [rows, cols] matrices with row strides in elements (multiples of 16 bytes): gate and up are the two
+ * column halves of ONE projection output (gate_proj and up_proj of models/llama.py:196-206 run as one GEMM over their
+ * adjacent weights), dgate and dup the halves of one gradient buffer, so that the next GEMM reads them without a copy. */
+int mlts_swiglu_fwd_rows(const void* gate, const void* up, int64_t ld_in, void* h, int64_t ld_h, int64_t rows, int64_t cols,
+                         int32_t dtype, mlts_stream_t stream);
+int mlts_swiglu_bwd_rows(const void* dh, int64_t ld_dh, const void* gate, const void* up, int64_t ld_in, void* dgate, void* dup,
+                         int64_t ld_out, int64_t rows, int64_t cols, int32_t dtype, mlts_stream_t stream);
+
 /* Causal cross-entropy, forward and gradient in one pass over the logits (utils/losses.py:9-15):
  *   loss = sum_{t: label_t != ignore_index} (logsumexp(z_t) - z_t[label_t]) / max(1, #targets)
  *   dlogits_t = (softmax(z_t) - onehot(label_t)) / max(1, #targets) for supervised rows, else 0.

@@ -100,6 +100,8 @@ SIGNATURES: dict[str, tuple[object, list[object]]] = {
     ),
     "mlts_swiglu_fwd": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, _P]),
     "mlts_swiglu_bwd": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int32, _P]),
+    "mlts_swiglu_fwd_rows": (C.c_int, [_P, _P, C.c_int64, _P, C.c_int64, C.c_int64, C.c_int64, C.c_int32, _P]),
+    "mlts_swiglu_bwd_rows": (C.c_int, [_P, C.c_int64, _P, _P, C.c_int64, _P, _P, C.c_int64, C.c_int64, C.c_int64, C.c_int32, _P]),
     "mlts_ce_workspace_bytes": (C.c_int64, [C.c_int64]),
     "mlts_ce_fwd_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int32, C.c_int64, C.c_int32, _P]),
     "mlts_scale_by_device_scalar": (C.c_int, [_P, _P, C.c_int64, C.c_int32, _P]),

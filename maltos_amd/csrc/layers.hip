@@ -4,6 +4,8 @@
 // are the reference's values and not merely close to them.
 #include "common.hpp"
 
+#include <initializer_list>
+
 // The kernels below reproduce the reference's per-op bf16 roundings.  With contraction enabled the
 // compiler narrows "round(a * b)" to a bf16 multiply and then fuses it into the following add as an
 // fp32 FMA, which silently drops that rounding; contraction stays off for this whole file.
@@ -341,6 +343,51 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const T* __restric
   }
 }
 
+// The same two kernels over [rows, cols] matrices with row strides (in elements, multiples of the vector width): gate
+// and up are the two column halves of one projection output, dgate and dup those of one gradient buffer.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_fwd_rows_kernel(const T* __restrict__ gate, const T* __restrict__ up, int64_t ld_in,
+                                                                   T* __restrict__ h, int64_t ld_h, uint32_t vec_per_row, uint32_t nvec) {
+  constexpr int N = Vec16<T>::N;
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+    const uint32_t row = i / vec_per_row, c = i - row * vec_per_row;
+    const int64_t in = static_cast<int64_t>(row) * ld_in + c * N;
+    Vec16<T> g = *reinterpret_cast<const Vec16<T>*>(gate + in);
+    Vec16<T> u = *reinterpret_cast<const Vec16<T>*>(up + in);
+    Vec16<T> o;
+#pragma unroll
+    for (int j = 0; j < N; ++j) o.set(j, round_to<T>(siluf_(g.get(j))) * u.get(j));
+    *reinterpret_cast<Vec16<T>*>(h + static_cast<int64_t>(row) * ld_h + c * N) = o;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_rows_kernel(const T* __restrict__ dh, int64_t ld_dh, const T* __restrict__ gate,
+                                                                   const T* __restrict__ up, int64_t ld_in, T* __restrict__ dgate,
+                                                                   T* __restrict__ dup, int64_t ld_out, uint32_t vec_per_row,
+                                                                   uint32_t nvec) {
+  constexpr int N = Vec16<T>::N;
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+    const uint32_t row = i / vec_per_row, c = i - row * vec_per_row;
+    const int64_t in = static_cast<int64_t>(row) * ld_in + c * N, out = static_cast<int64_t>(row) * ld_out + c * N;
+    Vec16<T> d = *reinterpret_cast<const Vec16<T>*>(dh + static_cast<int64_t>(row) * ld_dh + c * N);
+    Vec16<T> g = *reinterpret_cast<const Vec16<T>*>(gate + in);
+    Vec16<T> u = *reinterpret_cast<const Vec16<T>*>(up + in);
+    Vec16<T> og, ou;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+      const float gj = g.get(j), dj = d.get(j);
+      const float sg = sigmoidf_(gj);
+      ou.set(j, dj * (gj * sg));
+      og.set(j, dj * u.get(j) * (sg * (1.0f + gj * (1.0f - sg))));
+    }
+    *reinterpret_cast<Vec16<T>*>(dgate + out) = og;
+    *reinterpret_cast<Vec16<T>*>(dup + out) = ou;
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void swiglu_fwd_tail(const T* gate, const T* up, T* h, int64_t start, int64_t n) {
   int64_t i = start + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -670,4 +717,53 @@ extern "C" int mlts_swiglu_bwd(const void* dh, const void* gate, const void* up,
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == MLTS_BF16 ? swiglu_bwd_t<bf16_t>(dh, gate, up, dgate, dup, n, vec, st)
                             : swiglu_bwd_t<float>(dh, gate, up, dgate, dup, n, vec, st);
+}
+
+namespace {
+int swiglu_rows_check(const char* who, int64_t rows, int64_t cols, int32_t dtype, std::initializer_list<const void*> ptrs,
+                      std::initializer_list<int64_t> lds) {
+  MLTS_REQUIRE(known_dtype(dtype), "%s: unknown dtype %d", who, dtype);
+  const int n = elem_per_vec(dtype);
+  MLTS_REQUIRE(rows >= 0 && cols >= 0 && cols % n == 0, "%s: cols=%lld must be a multiple of %d", who, (long long)cols, n);
+  MLTS_REQUIRE(rows * (cols / n) < (int64_t{1} << 31), "%s: rows * cols too large", who);
+  for (const void* q : ptrs) MLTS_REQUIRE(rows * cols == 0 || (q && mlts_aligned16(q)), "%s: null or unaligned pointer", who);
+  for (int64_t ld : lds) MLTS_REQUIRE(ld >= cols && ld % n == 0, "%s: row strides must be >= cols and multiples of %d", who, n);
+  return MLTS_OK;
+}
+}  // namespace
+
+extern "C" int mlts_swiglu_fwd_rows(const void* gate, const void* up, int64_t ld_in, void* h, int64_t ld_h, int64_t rows,
+                                    int64_t cols, int32_t dtype, mlts_stream_t stream) {
+  if (int rc = swiglu_rows_check("mlts_swiglu_fwd_rows", rows, cols, dtype, {gate, up, h}, {ld_in, ld_h}); rc != MLTS_OK) return rc;
+  if (rows * cols == 0) return MLTS_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MltsKernelTimer timer("swiglu_fwd", st);
+  const uint32_t vpr = static_cast<uint32_t>(cols / elem_per_vec(dtype)), nvec = static_cast<uint32_t>(rows) * vpr;
+  if (dtype == MLTS_BF16)
+    hipLaunchKernelGGL(swiglu_fwd_rows_kernel<bf16_t>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const bf16_t*>(gate),
+                       static_cast<const bf16_t*>(up), ld_in, static_cast<bf16_t*>(h), ld_h, vpr, nvec);
+  else
+    hipLaunchKernelGGL(swiglu_fwd_rows_kernel<float>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const float*>(gate),
+                       static_cast<const float*>(up), ld_in, static_cast<float*>(h), ld_h, vpr, nvec);
+  return mlts_check_launch("mlts_swiglu_fwd_rows");
+}
+
+extern "C" int mlts_swiglu_bwd_rows(const void* dh, int64_t ld_dh, const void* gate, const void* up, int64_t ld_in, void* dgate,
+                                    void* dup, int64_t ld_out, int64_t rows, int64_t cols, int32_t dtype, mlts_stream_t stream) {
+  if (int rc = swiglu_rows_check("mlts_swiglu_bwd_rows", rows, cols, dtype, {dh, gate, up, dgate, dup}, {ld_dh, ld_in, ld_out});
+      rc != MLTS_OK)
+    return rc;
+  if (rows * cols == 0) return MLTS_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MltsKernelTimer timer("swiglu_bwd", st);
+  const uint32_t vpr = static_cast<uint32_t>(cols / elem_per_vec(dtype)), nvec = static_cast<uint32_t>(rows) * vpr;
+  if (dtype == MLTS_BF16)
+    hipLaunchKernelGGL(swiglu_bwd_rows_kernel<bf16_t>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const bf16_t*>(dh),
+                       ld_dh, static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up), ld_in, static_cast<bf16_t*>(dgate),
+                       static_cast<bf16_t*>(dup), ld_out, vpr, nvec);
+  else
+    hipLaunchKernelGGL(swiglu_bwd_rows_kernel<float>, dim3(stream_grid(nvec)), dim3(kThreads), 0, st, static_cast<const float*>(dh), ld_dh,
+                       static_cast<const float*>(gate), static_cast<const float*>(up), ld_in, static_cast<float*>(dgate),
+                       static_cast<float*>(dup), ld_out, vpr, nvec);
+  return mlts_check_launch("mlts_swiglu_bwd_rows");
 }

@@ -44,6 +44,11 @@ class LlamaConfig:
     # buffer of their size).  Nobody else may then read the lm_head output of that forward; the model falls back to a
     # separate gradient buffer by itself while lm_head carries forward hooks (which see that output).  False: always separate
     loss_overwrites_logits: bool = True
+    # q/k/v (and gate/up) projections run as one product whenever their weights are adjacent in memory (flat optimizer
+    # layouts); the sums inside that product are formed in another order than in three separate ones, so results differ
+    # from the separate form in the last bit.  False (or `module.fuse_projections = False` on an attention / MLP module)
+    # keeps one product per projection
+    fuse_projections: bool = True
 
     def __post_init__(self) -> None:
         validate_attention_backend(self.attention_backend)
@@ -60,6 +65,24 @@ def _weight_grad_splits(rows: int, out_features: int, in_features: int) -> int:
     return splits
 
 
+def _weight_grad(x2: torch.Tensor, dy2: torch.Tensor, grad: torch.Tensor | None) -> torch.Tensor | None:
+    """dW = dy2^T x2 for [rows, out] / [rows, in] operands, as a batch of row-slice products where that fills the chip
+    better.  With `grad` (the gradient buffer the weight already owns, a view of a flat gradient buffer) dW is added
+    into it in the pass that finishes it and None is returned; otherwise dW is returned."""
+    splits = _weight_grad_splits(x2.shape[0], dy2.shape[1], x2.shape[1])
+    if splits > 1 and x2.is_contiguous() and dy2.is_contiguous():
+        rows = x2.shape[0] // splits
+        part = torch.bmm(dy2.view(splits, rows, -1).transpose(1, 2), x2.view(splits, rows, -1))
+        if grad is not None:
+            ops.grad_sum_slices(part, grad, accumulate=True)    # fp32 sum of slices + old grad, rounded once
+            return None
+        return ops.grad_sum_slices(part)                        # slices added in fp32, rounded once
+    if grad is not None:
+        grad.addmm_(dy2.t(), x2)
+        return None
+    return dy2.t().matmul(x2)
+
+
 class _SplitKLinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x: torch.Tensor, weight: torch.Tensor, into_grad: bool) -> torch.Tensor:
@@ -74,28 +97,125 @@ class _SplitKLinearFn(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = dy.matmul(weight)
         if ctx.needs_input_grad[1]:
-            x2 = x.reshape(-1, x.shape[-1])
-            dy2 = dy.reshape(-1, dy.shape[-1])
-            # the gradient buffer this weight already owns (a view of a flat gradient buffer): add into it here, in
-            # the pass that finishes dW, instead of handing dW to autograd for a separate `grad += dW`
             grad = weight.grad if ctx.into_grad else None
             if grad is not None and not (grad.is_contiguous() and grad.dtype == weight.dtype and grad.shape == weight.shape):
                 grad = None
-            splits = _weight_grad_splits(x2.shape[0], dy2.shape[1], x2.shape[1])
-            if splits > 1 and x2.is_contiguous() and dy2.is_contiguous():
-                rows = x2.shape[0] // splits
-                part = torch.bmm(dy2.view(splits, rows, -1).transpose(1, 2), x2.view(splits, rows, -1))
-                if grad is not None:
-                    ops.grad_sum_slices(part, grad, accumulate=True)    # fp32 sum of slices + old grad, rounded once
-                else:
-                    dw = ops.grad_sum_slices(part)                      # slices added in fp32, rounded once
-            elif grad is not None:
-                grad.addmm_(dy2.t(), x2)
-            else:
-                dw = dy2.t().matmul(x2)
+            dw = _weight_grad(x.reshape(-1, x.shape[-1]), dy.reshape(-1, dy.shape[-1]), grad)
             if grad is not None:
                 notify_grad_written(weight)   # autograd's hooks on the weight do not fire for a gradient added here
         return dx, dw, None
+
+
+# ---- projections that share their input, run as ONE GEMM over adjacent weights ------------------------------------
+# q_proj / k_proj / v_proj (and gate_proj / up_proj) read the same activations.  When their weights are adjacent row
+# blocks of one allocation (what the flat optimizer layouts make of them: MasterWeightsOptimizer(flat=True),
+# Zero1FlatBuffers), they ARE one [sum of out_features, in_features] matrix, and the three (two) products are one: at
+# LLaMA-50M sizes a 512-wide product has 128 output tiles for 256 compute units, the 1536-wide one fills the chip, and
+# the backward's three input-gradient products and their two additions become one product.  Parameter names, shapes
+# and values are untouched; without adjacency the projections run one by one as in the reference (models/llama.py:
+# 134-142,196-206).
+class _FusedRows:
+    """Adjacent 2-D parameters seen as one matrix: `weight` [R, in] and, when their .grad views are adjacent in the same
+    order, `grad` [R, in]; `cols[i]` = (first, last + 1) output column of parameter i (caller order)."""
+
+    __slots__ = ("key", "weight", "grad", "cols")
+
+
+def _fused_rows(holder: nn.Module, params: list[nn.Parameter]) -> _FusedRows | None:
+    key = tuple((p.data_ptr(), 0 if p.grad is None else p.grad.data_ptr()) for p in params)
+    cached = holder.__dict__.get("_maltos_hip_fused_rows")
+    if cached is not None and cached.key == key:
+        return cached if cached.weight is not None else None
+    fused = _FusedRows()
+    fused.key, fused.weight, fused.grad, fused.cols = key, None, None, []
+    holder.__dict__["_maltos_hip_fused_rows"] = fused
+    first = params[0]
+    if not all(p.dim() == 2 and p.is_cuda and p.is_contiguous() and p.dtype == first.dtype and p.size(1) == first.size(1)
+               and p.requires_grad for p in params):
+        return None
+    order = sorted(range(len(params)), key=lambda i: params[i].data_ptr())
+    es = first.element_size()
+    for a, b in zip(order, order[1:]):
+        pa, pb = params[a], params[b]
+        if pa.untyped_storage().data_ptr() != pb.untyped_storage().data_ptr() or pa.data_ptr() + pa.numel() * es != pb.data_ptr():
+            return None
+    rows = sum(p.size(0) for p in params)
+    base = params[order[0]]
+    fused.weight = base.data.as_strided((rows, base.size(1)), (base.size(1), 1))
+    start, cols = 0, [None] * len(params)
+    for i in order:
+        cols[i] = (start, start + params[i].size(0))
+        start += params[i].size(0)
+    fused.cols = cols
+    grads = [p.grad for p in params]
+    if all(g is not None and g.is_contiguous() and g.dtype == first.dtype and g.shape == p.shape for g, p in zip(grads, params)):
+        if all(grads[a].untyped_storage().data_ptr() == grads[b].untyped_storage().data_ptr()
+               and grads[a].data_ptr() + grads[a].numel() * es == grads[b].data_ptr() for a, b in zip(order, order[1:])):
+            g0 = grads[order[0]]
+            fused.grad = g0.as_strided((rows, g0.size(1)), (g0.size(1), 1))
+    return fused
+
+
+def _fusable(modules: list[nn.Module]) -> bool:
+    return all(isinstance(m, HipLinear) and m.bias is None for m in modules)
+
+
+class _FusedLinearsFn(torch.autograd.Function):
+    """(x W_0^T, x W_1^T, ...) from one product with the parameters' common matrix; the outputs are column slices of it."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, fused: _FusedRows, into_grad: bool, *weights: torch.Tensor):
+        ctx.save_for_backward(x)
+        ctx.fused, ctx.into_grad, ctx.weights = fused, into_grad and fused.grad is not None, weights
+        y = F.linear(x, fused.weight)
+        return tuple(y[..., a:b] for a, b in fused.cols)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        (x,) = ctx.saved_tensors
+        fused = ctx.fused
+        rows_total = fused.weight.size(0)
+        x2 = x.reshape(-1, x.shape[-1])
+        # the slices' gradients side by side, in the order of the rows of the common matrix
+        dy2 = torch.empty((x2.shape[0], rows_total), dtype=x.dtype, device=x.device)
+        for (a, b), dy in zip(fused.cols, dys):
+            if dy is None:
+                dy2[:, a:b].zero_()
+            else:
+                dy2[:, a:b].copy_(dy.reshape(-1, b - a))
+        dx = dy2.matmul(fused.weight).view(x.shape) if ctx.needs_input_grad[0] else None
+        dw = _weight_grad(x2, dy2, fused.grad if ctx.into_grad else None)
+        if dw is None:
+            for w in ctx.weights:
+                notify_grad_written(w)
+            return (dx, None, None, *([None] * len(ctx.weights)))
+        return (dx, None, None, *(dw[a:b] for a, b in fused.cols))
+
+
+class _FusedGateUpFn(torch.autograd.Function):
+    """round(silu(x W_gate^T)) * (x W_up^T) (models/llama.py:205-206) with the two projections as one product; the
+    backward writes d gate and d up side by side, so that the input gradient is one product as well."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, fused: _FusedRows, into_grad: bool, w_gate: torch.Tensor, w_up: torch.Tensor):
+        gu = F.linear(x, fused.weight)
+        ctx.save_for_backward(x, gu)
+        ctx.fused, ctx.into_grad, ctx.weights = fused, into_grad and fused.grad is not None, (w_gate, w_up)
+        return ops.swiglu_rows(gu, fused.cols[0][0], fused.cols[1][0], w_gate.size(0))
+
+    @staticmethod
+    def backward(ctx, dh: torch.Tensor):
+        x, gu = ctx.saved_tensors
+        fused = ctx.fused
+        dgu = ops.swiglu_rows_backward(dh, gu, fused.cols[0][0], fused.cols[1][0], ctx.weights[0].size(0))
+        dgu2 = dgu.view(-1, dgu.shape[-1])
+        dx = dgu2.matmul(fused.weight).view(x.shape) if ctx.needs_input_grad[0] else None
+        dw = _weight_grad(x.reshape(-1, x.shape[-1]), dgu2, fused.grad if ctx.into_grad else None)
+        if dw is None:
+            for w in ctx.weights:
+                notify_grad_written(w)
+            return dx, None, None, None, None
+        return (dx, None, None, *(dw[a:b] for a, b in fused.cols))
 
 
 class HipLinear(nn.Linear):
@@ -188,6 +308,7 @@ class LlamaAttention(nn.Module):
         self.v_proj = HipLinear(config.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
         self.o_proj = HipLinear(config.hidden_size, config.hidden_size, bias=False)
         self.attn_core = HipAttentionCore(config.attention_backend)
+        self.fuse_projections = config.fuse_projections
 
     def forward(self, x: torch.Tensor, *, position_offset: int = 0, position_ids: torch.Tensor | None = None,
                 sequence_ids: torch.Tensor | None = None) -> torch.Tensor:
@@ -198,9 +319,18 @@ class LlamaAttention(nn.Module):
             rope_pos = canonical_position_ids(position_ids, batch_size=batch, seq_len=seq_len, position_offset=0,
                                               device=x.device)
         # [B, S, H*D] -> [B, H, S, D] views; no copies until the kernels read them
-        q = self.q_proj(x).view(batch, seq_len, self.num_heads, self.head_dim).transpose(1, 2)
-        k = self.k_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
-        v = self.v_proj(x).view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
+        projections = [self.q_proj, self.k_proj, self.v_proj]
+        fused = None
+        if self.fuse_projections and x.is_cuda and _fusable(projections):
+            fused = _fused_rows(self, [m.weight for m in projections])
+        if fused is not None:   # one product over the three adjacent weights
+            q, k, v = _FusedLinearsFn.apply(x, fused, all(m.accumulate_into_grad for m in projections),
+                                            *(m.weight for m in projections))
+        else:
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        q = q.view(batch, seq_len, self.num_heads, self.head_dim).transpose(1, 2)
+        k = k.view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
+        v = v.view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
         q, k = ops.rope_pair(q, k, cos, sin, positions=rope_pos, position_offset=position_offset)
         if not getattr(self.attn_core, "preserves_native_gqa", False) and self.num_heads != self.num_kv_heads:
             rep = self.num_heads // self.num_kv_heads
@@ -215,8 +345,16 @@ class LlamaMLP(nn.Module):
         self.gate_proj = HipLinear(config.hidden_size, config.intermediate_size, bias=False)
         self.up_proj = HipLinear(config.hidden_size, config.intermediate_size, bias=False)
         self.down_proj = HipLinear(config.intermediate_size, config.hidden_size, bias=False)
+        self.fuse_projections = config.fuse_projections
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        pair = [self.gate_proj, self.up_proj]
+        fused = None
+        if self.fuse_projections and x.is_cuda and _fusable(pair) and self.gate_proj.out_features % (16 // x.element_size()) == 0:
+            fused = _fused_rows(self, [m.weight for m in pair])
+        if fused is not None:
+            h = _FusedGateUpFn.apply(x, fused, all(m.accumulate_into_grad for m in pair), self.gate_proj.weight, self.up_proj.weight)
+            return self.down_proj(h)
         return self.down_proj(ops.swiglu(self.gate_proj(x), self.up_proj(x)))
 
 

@@ -431,6 +431,37 @@ def _swiglu_bwd(dh, gate, up):
     return dg, du
 
 
+def swiglu_rows(gu: torch.Tensor, gate_col: int, up_col: int, cols: int) -> torch.Tensor:
+    """round(silu(gate)) * up where gate = gu[..., gate_col : gate_col + cols] and up = gu[..., up_col : up_col + cols] are
+    column blocks of one contiguous [..., width] projection output (no autograd: used inside the fused MLP function)."""
+    _require_gpu(gu)
+    if not gu.is_contiguous():
+        raise ValueError("swiglu_rows expects a contiguous projection output")
+    width = gu.size(-1)
+    rows = gu.numel() // width
+    h = torch.empty((*gu.shape[:-1], cols), dtype=gu.dtype, device=gu.device)
+    es = gu.element_size()
+    _lib.check(_lib.lib().mlts_swiglu_fwd_rows(C.c_void_p(gu.data_ptr() + gate_col * es), C.c_void_p(gu.data_ptr() + up_col * es), width,
+                                               _p(h), cols, rows, cols, _dtype_code(gu), _stream()))
+    return h
+
+
+def swiglu_rows_backward(dh: torch.Tensor, gu: torch.Tensor, gate_col: int, up_col: int, cols: int) -> torch.Tensor:
+    """d gate and d up of swiglu_rows, written into the same column blocks of a buffer shaped like `gu`; its other
+    columns, if there are any, are zero."""
+    _require_gpu(dh, gu)
+    dh = dh.contiguous()
+    width = gu.size(-1)
+    rows = gu.numel() // width
+    dgu = torch.empty_like(gu) if width == 2 * cols else torch.zeros_like(gu)
+    es = gu.element_size()
+    _lib.check(_lib.lib().mlts_swiglu_bwd_rows(_p(dh), cols, C.c_void_p(gu.data_ptr() + gate_col * es),
+                                               C.c_void_p(gu.data_ptr() + up_col * es), width,
+                                               C.c_void_p(dgu.data_ptr() + gate_col * es), C.c_void_p(dgu.data_ptr() + up_col * es), width,
+                                               rows, cols, _dtype_code(gu), _stream()))
+    return dgu
+
+
 def _ce_fwd_bwd(logits, labels, ignore_index, overwrite: bool = False):
     """overwrite: the gradient replaces the logits in their own buffer (they must be contiguous)."""
     _require_gpu(logits, labels)
