@@ -177,12 +177,16 @@ class _FusedLinearsFn(torch.autograd.Function):
         rows_total = fused.weight.size(0)
         x2 = x.reshape(-1, x.shape[-1])
         # the slices' gradients side by side, in the order of the rows of the common matrix
-        dy2 = torch.empty((x2.shape[0], rows_total), dtype=x.dtype, device=x.device)
-        for (a, b), dy in zip(fused.cols, dys):
-            if dy is None:
-                dy2[:, a:b].zero_()
-            else:
-                dy2[:, a:b].copy_(dy.reshape(-1, b - a))
+        order = sorted(range(len(dys)), key=lambda i: fused.cols[i][0])
+        if all(dy is not None for dy in dys):
+            dy2 = torch.cat([dys[i].reshape(-1, fused.cols[i][1] - fused.cols[i][0]) for i in order], dim=1)  # one launch
+        else:
+            dy2 = torch.empty((x2.shape[0], rows_total), dtype=x.dtype, device=x.device)
+            for (a, b), dy in zip(fused.cols, dys):
+                if dy is None:
+                    dy2[:, a:b].zero_()
+                else:
+                    dy2[:, a:b].copy_(dy.reshape(-1, b - a))
         dx = dy2.matmul(fused.weight).view(x.shape) if ctx.needs_input_grad[0] else None
         dw = _weight_grad(x2, dy2, fused.grad if ctx.into_grad else None)
         if dw is None:
