@@ -127,8 +127,10 @@ def test_document_mask_many_tiles(dev, D):
 
 @pytest.mark.parametrize("D", [64, 128])
 def test_document_mask_long_row_equals_causal_attention_per_document(dev, D):
-    """A size the oracle does not reach (32768 tokens): packed documents attend exactly as each document alone under the
-    causal mask, forward and backward, so the document kernels are checked against the causal kernels slice by slice."""
+    """A size the oracle does not reach as a whole (32768 tokens): packed documents attend exactly as each document alone
+    under the causal mask, forward and backward, so the document kernels are checked against the causal kernels slice by
+    slice, and the slices short enough for the oracle (up to 4097 tokens, at the start, in the middle and at the end of
+    the row) against the oracle itself."""
     S, Hq, Hkv = 32768, 4, 2
     gen = torch.Generator().manual_seed(7 + D)
     q, k, v, do = (bshd(1, h, S, D, gen, torch.bfloat16).to(dev) for h in (Hq, Hkv, Hkv, Hq))
@@ -147,6 +149,14 @@ def test_document_mask_long_row_equals_causal_attention_per_document(dev, D):
         assert (lse[:, :, a:b] - lse1).abs().max() <= 4e-3, tag + " LSE (two kernel results, each within 2e-3)"
         for got, want, name in zip((dq, dk, dv), g1, ("dQ", "dK", "dV")):
             check(got[sl], want, torch.bfloat16, f"{tag} {name}")
+        if b - a <= 4097:
+            qc, kc, vc, dc = (t[sl].float().cpu() for t in (q, k, v, do))
+            want_o, want_lse = oa.attention_with_lse(qc, kc, vc, oa.causal_mask(b - a, b - a, "cpu"))
+            check(o[sl], want_o, torch.bfloat16, tag + " O against the oracle")
+            assert (lse[:, :, a:b].cpu() - want_lse).abs().max() <= 2e-3, tag + " LSE against the oracle"
+            wants = oa.attention_backward_explicit(dc, qc, kc, vc, want_o, want_lse, oa.causal_mask(b - a, b - a, "cpu"))
+            for got, want, name in zip((dq, dk, dv), wants, ("dQ", "dK", "dV")):
+                check(got[sl], want, torch.bfloat16, f"{tag} {name} against the oracle")
 
 
 @pytest.mark.parametrize("seed", range(10))
