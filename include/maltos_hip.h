@@ -190,7 +190,8 @@ int mlts_add_rmsnorm_bwd(const void* dy, const void* x, const void* w, const flo
  * every product and the sum rounded to `dtype` as the reference's eager ops do.
  * x, y: [B, H, S, D] with element strides (batch, head, seq); cos/sin: [max_pos, D/2] of `dtype`.
  * positions: int32 [B, S] or NULL (then pos = position_offset + s).  inverse != 0 rotates by
- * -theta, which is the backward pass. */
+ * -theta, which is the backward pass.  y may be x with the same strides (rotation in place); any other overlap of the
+ * two is undefined. */
 int mlts_rope(const void* x, const int64_t x_stride[3], void* y, const int64_t y_stride[3], const void* cos_tab,
               const void* sin_tab, int32_t max_pos, const int32_t* positions, int32_t position_offset,
               int32_t B, int32_t H, int32_t S, int32_t D, int32_t dtype, int32_t inverse,

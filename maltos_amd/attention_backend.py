@@ -47,6 +47,11 @@ def validate_attention_backend(attention_backend: "str | AttentionBackend") -> A
         ) from None
 
 
+def uses_hip_kernels(attention_backend: str) -> bool:
+    """Whether this backend name routes to the hand-written kernels (the others evaluate attention with torch ops)."""
+    return validate_attention_backend(attention_backend) in _HIP_BACKENDS
+
+
 def hip_fallback_reason(q: torch.Tensor) -> str | None:
     """None when the HIP kernels can take `q`, else why not (reference: flash_attn_fallback_reason,
     runtime/layers/flash_utils.py:105-115).  The router raises with this string instead of degrading."""

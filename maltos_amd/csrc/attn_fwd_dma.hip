@@ -487,11 +487,11 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
       }
       const float m_use = m_run == -INFINITY ? 0.f : m_run;
       if constexpr (D == 64) {
-        // probabilities in pairs: one packed conversion and one dot product with (1, 1) per pair, so the row sum is
-        // the sum of the bf16 values that enter the PV product (measured: 5 % faster at head_dim 64, 4 % slower at
-        // 128, which keeps the plain sum below)
+        // probabilities in pairs: one packed conversion per pair.  The row sum is taken over the fp32 values, not over
+        // the bf16 ones that enter the PV product: a dot product of each converted pair with (1, 1) is one instruction
+        // less per pair, but a bf16 value is off by up to 2^-8 of itself, and in a row that a few keys dominate that
+        // error goes straight into LSE (up to 4e-3, where the fp32 sum keeps it near 1e-6)
         float ls4[4] = {0.f, 0.f, 0.f, 0.f};
-        const bf16x2 ones = {static_cast<bf16_t>(1.0f), static_cast<bf16_t>(1.0f)};
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(THREADS) void attn_fwd_dma_kernel(const AttnParams 
               pv[0] = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + 2 * i] * p.scale_log2 - m_use);
               pv[1] = __builtin_amdgcn_exp2f(sacc[kb][t * 8 + 2 * i + 1] * p.scale_log2 - m_use);
               const bf16x2 pb = __builtin_convertvector(pv, bf16x2);
-              ls4[i] = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, ls4[i], false);
+              ls4[i] += pv[0] + pv[1];
               w[i] = __builtin_bit_cast(int, pb);
             }
             pf[kb * 2 + t] = __builtin_bit_cast(bf16x8, w);

@@ -220,9 +220,10 @@ int rmsnorm_bwd_blocks(int64_t rows) {
 // One lane rotates the pairs inside one 16-byte vector of a [b, h, s, :] row.
 // IDX is the type the flat element index is taken apart in: 32-bit whenever the tensor has fewer than 2^31 vectors
 // (three 64-bit divisions per lane cost several hundred instructions, more than the rotation itself).
+// y may be x (rotation in place: a lane reads only the vector it writes), so the two carry no __restrict__.
 template <typename T, bool INVERSE, typename IDX>
-__device__ __forceinline__ void rope_rows(const int64_t idx64, const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
-                                          T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
+__device__ __forceinline__ void rope_rows(const int64_t idx64, const T* x, int64_t xsb, int64_t xsh, int64_t xss,
+                                          T* y, int64_t ysb, int64_t ysh, int64_t yss,
                                           const T* __restrict__ cos_tab, const T* __restrict__ sin_tab, int max_pos,
                                           const int32_t* __restrict__ positions, int position_offset, int B, int H, int S,
                                           int D) {
@@ -268,8 +269,8 @@ __device__ __forceinline__ void rope_rows(const int64_t idx64, const T* __restri
 }
 
 template <typename T, bool INVERSE, typename IDX>
-__global__ __launch_bounds__(kThreads) void rope_kernel(const T* __restrict__ x, int64_t xsb, int64_t xsh, int64_t xss,
-                                                        T* __restrict__ y, int64_t ysb, int64_t ysh, int64_t yss,
+__global__ __launch_bounds__(kThreads) void rope_kernel(const T* x, int64_t xsb, int64_t xsh, int64_t xss,
+                                                        T* y, int64_t ysb, int64_t ysh, int64_t yss,
                                                         const T* __restrict__ cos_tab, const T* __restrict__ sin_tab,
                                                         int max_pos, const int32_t* __restrict__ positions,
                                                         int position_offset, int B, int H, int S, int D) {

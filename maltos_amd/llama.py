@@ -16,7 +16,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .attention_backend import AttentionBackend, causal_attention, validate_attention_backend
+from .attention_backend import AttentionBackend, causal_attention, hip_fallback_reason, uses_hip_kernels, validate_attention_backend
 from .attn_masking_utils import canonical_position_ids, canonical_sequence_ids
 from .constants import (HIDDEN_STATES_KEY, INPUT_IDS_KEY, LABELS_KEY, LOSS_WEIGHT_KEY, POSITION_IDS_KEY,
                         POSITION_OFFSET_KEY, SEQUENCE_IDS_KEY)
@@ -156,6 +156,29 @@ def _fused_rows(holder: nn.Module, params: list[nn.Parameter]) -> _FusedRows | N
     return fused
 
 
+def _adjacent_columns(parts: list[torch.Tensor]) -> torch.Tensor | None:
+    """The [rows, sum of widths] matrix whose column ranges the given [..., width_i] tensors are, in this order, when
+    they are such views of one dense buffer; None otherwise (then the caller copies them together)."""
+    first = parts[0]
+    lead = first.shape[:-1]
+    total = sum(p.size(-1) for p in parts)
+    want, step = [], total
+    for n in reversed(lead):   # strides of a dense [*lead, total] buffer
+        want.append(step)
+        step *= n
+    want = tuple(reversed(want)) + (1,)
+    storage, offset = first.untyped_storage().data_ptr(), first.storage_offset()
+    for p in parts:
+        if (p.shape[:-1] != lead or p.dtype != first.dtype or p.untyped_storage().data_ptr() != storage
+                or p.storage_offset() != offset or any(n > 1 and a != b for n, a, b in zip(p.shape, p.stride(), want))):
+            return None
+        offset += p.size(-1)
+    rows = 1
+    for n in lead:
+        rows *= n
+    return first.as_strided((rows, total), (total, 1), first.storage_offset())
+
+
 def _fusable(modules: list[nn.Module]) -> bool:
     return all(isinstance(m, HipLinear) and m.bias is None for m in modules)
 
@@ -179,7 +202,9 @@ class _FusedLinearsFn(torch.autograd.Function):
         # the slices' gradients side by side, in the order of the rows of the common matrix
         order = sorted(range(len(dys)), key=lambda i: fused.cols[i][0])
         if all(dy is not None for dy in dys):
-            dy2 = torch.cat([dys[i].reshape(-1, fused.cols[i][1] - fused.cols[i][0]) for i in order], dim=1)  # one launch
+            dy2 = _adjacent_columns([dys[i] for i in order])   # already side by side (attention's joint gradient buffer)?
+            if dy2 is None:
+                dy2 = torch.cat([dys[i].reshape(-1, fused.cols[i][1] - fused.cols[i][0]) for i in order], dim=1)  # one launch
         else:
             dy2 = torch.empty((x2.shape[0], rows_total), dtype=x.dtype, device=x.device)
             for (a, b), dy in zip(fused.cols, dys):
@@ -285,18 +310,56 @@ class HipAttentionCore(nn.Module):
         super().__init__()
         self.attention_backend = validate_attention_backend(attention_backend)
 
+    def row_ids(self, q, position_offset: int, position_ids=None, sequence_ids=None):
+        """(positions, sequence ids) of the rows as the attention kernels take them, or (None, None) for plain causal rows."""
+        if position_ids is None and sequence_ids is None:
+            return None, None
+        positions = canonical_position_ids(position_ids, batch_size=q.size(0), seq_len=q.size(-2),
+                                           position_offset=position_offset, device=q.device)
+        return positions, canonical_sequence_ids(sequence_ids, batch_size=q.size(0), seq_len=q.size(-2), device=q.device)
+
     def forward(self, q, k, v, position_offset: int, position_ids=None, sequence_ids=None) -> torch.Tensor:
-        positions = sequences = None
-        if position_ids is not None or sequence_ids is not None:
-            positions = canonical_position_ids(position_ids, batch_size=q.size(0), seq_len=q.size(-2),
-                                               position_offset=position_offset, device=q.device)
-            sequences = canonical_sequence_ids(sequence_ids, batch_size=q.size(0), seq_len=q.size(-2), device=q.device)
+        positions, sequences = self.row_ids(q, position_offset, position_ids, sequence_ids)
         return causal_attention(q, k, v, attention_backend=self.attention_backend, warning_prefix="LlamaAttention",
                                 q_positions=positions, k_positions=positions, q_sequence_ids=sequences,
                                 k_sequence_ids=sequences, flash_varlen_mode="same_length")
 
 
+class _RopeAttentionFn(torch.autograd.Function):
+    """attention(rotary(q), rotary(k), v) (models/llama.py:143-150) as one autograd node over the same kernels as the
+    separate ops, hence the same values.  What the node adds is the layout of its backward: dQ, dK and dV are head ranges
+    of one [B, S, Hq + 2 Hkv, D] buffer and the rotation of dQ / dK back is done in place there (the buffer is the node's
+    own until it returns), so the gradient of q/k/v projections that run as one product arrives as one matrix."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cos, sin, rope_positions, position_offset: int, positions, sequences):
+        q, k = torch.ops.maltos.rope_pair(q, k, cos, sin, rope_positions, position_offset, False)
+        mask_mode = ops.MASK_CAUSAL
+        if positions is not None:
+            mask_mode = ops.MASK_DOC
+            if sequences is None:   # positions only: one document per row (the zero ids are kept with the positions)
+                sequences = ops.derived_from(positions, "_maltos_hip_zero_ids",
+                                             lambda pos: torch.zeros(pos.shape, dtype=torch.int32, device=pos.device))
+        out, lse = ops.attention_forward(q, k, v, mask_mode=mask_mode, q_pos=positions, k_pos=positions, q_seq=sequences,
+                                         k_seq=sequences)
+        ctx.save_for_backward(q, k, v, out, lse, cos, sin, rope_positions, positions, sequences)
+        ctx.position_offset, ctx.mask_mode = position_offset, mask_mode
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, cos, sin, rope_positions, positions, sequences = ctx.saved_tensors
+        dq, dk, dv = ops.attention_backward(dout, q, k, v, out, lse, mask_mode=ctx.mask_mode, q_pos=positions,
+                                            k_pos=positions, q_seq=sequences, k_seq=sequences)
+        ops.rope_pair_(dq, dk, cos, sin, positions=rope_positions, position_offset=ctx.position_offset, inverse=True)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
 class LlamaAttention(nn.Module):
+    # rotary embedding and attention as one autograd node whenever `attn_core` is the stock HipAttentionCore on the HIP
+    # kernels (same values; see _RopeAttentionFn).  False keeps the two ops apart
+    fuse_rope_attention = True
+
     def __init__(self, config: LlamaConfig) -> None:
         super().__init__()
         if config.hidden_size % config.num_attention_heads != 0:
@@ -335,6 +398,12 @@ class LlamaAttention(nn.Module):
         q = q.view(batch, seq_len, self.num_heads, self.head_dim).transpose(1, 2)
         k = k.view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
         v = v.view(batch, seq_len, self.num_kv_heads, self.head_dim).transpose(1, 2)
+        core = self.attn_core
+        if (self.fuse_rope_attention and type(core) is HipAttentionCore and uses_hip_kernels(core.attention_backend)
+                and hip_fallback_reason(q) is None):
+            positions, sequences = core.row_ids(q, position_offset, position_ids, sequence_ids)
+            vo = _RopeAttentionFn.apply(q, k, v, cos, sin, rope_pos, int(position_offset), positions, sequences)
+            return self.o_proj(vo.transpose(1, 2).reshape(batch, seq_len, self.num_heads * self.head_dim))
         q, k = ops.rope_pair(q, k, cos, sin, positions=rope_pos, position_offset=position_offset)
         if not getattr(self.attn_core, "preserves_native_gqa", False) and self.num_heads != self.num_kv_heads:
             rep = self.num_heads // self.num_kv_heads

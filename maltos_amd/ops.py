@@ -23,7 +23,7 @@ __all__ = [
     "MASK_NONE", "MASK_CAUSAL", "MASK_DOC",
     "attention", "attention_forward", "attention_backward", "attention_backward_accumulate",
     "attention_backward_ring_block", "attention_merge_",
-    "rms_norm", "rope", "rope_pair", "swiglu", "cross_entropy",
+    "rms_norm", "rope", "rope_pair", "rope_pair_", "swiglu", "cross_entropy",
     "adamw_step_", "sq_norm", "scale_", "grad_to_f32_",
 ]
 
@@ -251,11 +251,20 @@ def _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, accumulate, mask
 
 def attention_backward(dout, q, k, v, o, lse, *, mask_mode: int, scale: float | None = None, q_pos=None, k_pos=None,
                        q_seq=None, k_seq=None):
-    """(dq, dk, dv) in the input dtype, laid out like q, k, v."""
+    """(dq, dk, dv) in the input dtype, as [B, H, S, D] views of [B, S, H, D] storage.  For self-attention (queries and
+    keys of one length) the three are the head ranges [0, Hq), [Hq, Hq + Hkv), [Hq + Hkv, Hq + 2 Hkv) of ONE
+    [B, S, Hq + 2 Hkv, D] buffer: next to each other exactly as the input gradient of projections that run as one
+    product wants them, so that nobody has to copy them together."""
     q, k, v, o, dout = map(_dense_last, (q, k, v, o, dout))
-    dq = _bshd_empty(q.size(0), q.size(1), q.size(2), q.size(3), q)
-    dk = _bshd_empty(k.size(0), k.size(1), k.size(2), k.size(3), k)
-    dv = _bshd_empty(v.size(0), v.size(1), v.size(2), v.size(3), v)
+    B, Hq, Sq, D = q.shape
+    Hkv = k.size(1)
+    if k.size(2) == Sq and k.dtype == q.dtype and v.dtype == q.dtype:
+        joint = _bshd_empty(B, Hq + 2 * Hkv, Sq, D, q)
+        dq, dk, dv = joint[:, :Hq], joint[:, Hq:Hq + Hkv], joint[:, Hq + Hkv:]
+    else:
+        dq = _bshd_empty(B, Hq, Sq, D, q)
+        dk = _bshd_empty(k.size(0), Hkv, k.size(2), k.size(3), k)
+        dv = _bshd_empty(v.size(0), v.size(1), v.size(2), v.size(3), v)
     _attention_backward_impl(dout, q, k, v, o, lse, dq, dk, dv, BWD_OVERWRITE, mask_mode, scale, q_pos, k_pos, q_seq, k_seq)
     return dq, dk, dv
 
@@ -392,7 +401,7 @@ def _rope(x, cos, sin, positions, position_offset, inverse):
     return y
 
 
-def _rope_pair(xa, xb, cos, sin, positions, position_offset, inverse):
+def _rope_pair(xa, xb, cos, sin, positions, position_offset, inverse, in_place: bool = False):
     """Both rotations of an attention layer (query and key projections) in one launch."""
     _require_gpu(xa, xb, cos, sin, positions)
     if xa.dim() != 4 or xb.dim() != 4 or xa.size(0) != xb.size(0) or xa.shape[2:] != xb.shape[2:] or xa.dtype != xb.dtype:
@@ -402,8 +411,13 @@ def _rope_pair(xa, xb, cos, sin, positions, position_offset, inverse):
         raise ValueError(f"cos/sin tables must be [max_pos, {D // 2}], got {tuple(cos.shape)}")
     if cos.dtype != xa.dtype or sin.dtype != xa.dtype:
         raise ValueError("cos/sin tables must have the activation dtype (the reference casts them first)")
-    xa, xb = _dense_last(xa), _dense_last(xb)
-    ya, yb = torch.empty_like(xa), torch.empty_like(xb)
+    if in_place:
+        if xa.stride(-1) != 1 or xb.stride(-1) != 1:
+            raise ValueError("rope_pair_: the head_dim of both tensors must be contiguous")
+        ya, yb = xa, xb
+    else:
+        xa, xb = _dense_last(xa), _dense_last(xb)
+        ya, yb = torch.empty_like(xa), torch.empty_like(xb)
     pos32 = None if positions is None else _ids32(positions, B, S, "position_ids")
     cos, sin = cos.contiguous(), sin.contiguous()
     _lib.check(_lib.lib().mlts_rope_pair(_p(xa), strides3(xa.stride()[:3]), _p(ya), strides3(ya.stride()[:3]), Ha,
@@ -817,6 +831,13 @@ def rope_pair(xa: torch.Tensor, xb: torch.Tensor, cos: torch.Tensor, sin: torch.
               position_offset: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
     """rope(xa), rope(xb) from one kernel launch (and one in the backward): bit-equal to two `rope` calls."""
     return torch.ops.maltos.rope_pair(xa, xb, cos, sin, positions, int(position_offset), False)
+
+
+def rope_pair_(xa: torch.Tensor, xb: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, positions: torch.Tensor | None = None,
+               position_offset: int = 0, inverse: bool = False) -> None:
+    """`rope_pair` written over its inputs, outside autograd (`inverse` rotates back: the backward pass).  For buffers
+    the caller owns, e.g. the gradients an attention backward has just produced."""
+    _rope_pair(xa, xb, cos, sin, positions, int(position_offset), inverse, in_place=True)
 
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -8,7 +8,7 @@ Tolerances
       O, dQ, dK, dV : |err| <= 2e-2 + 2^-8 |want|.  2e-2 is the stated max-abs bar; the second term is half a
                       bf16 ulp of the expected value, the rounding any bf16 output carries (it matters only
                       for |want| > ~5, e.g. dV rows that sum many queries).
-      LSE (fp32)    : 2e-3 absolute.
+      LSE (fp32)    : 1e-4 absolute (scores and row sums are formed in fp32 from the bf16 inputs; measured ~4e-6).
   * reference ring test vectors (fp32, head_dim 3): forward 1e-5, backward 2e-5, the reference's own bars
     (zigzag ring and packed-document ring).
 """
@@ -77,7 +77,7 @@ def run_case(dev, dtype, B, Hq, Hkv, Sq, Sk, D, mode, seed, *, max_doc=None, pad
     check(o, want_o, dtype, tag + " O")
     fin = torch.isfinite(want_lse)
     assert torch.equal(torch.isfinite(lse.cpu()), fin), tag + " LSE -inf pattern"
-    lse_tol = 1e-4 if dtype == torch.float32 else 2e-3
+    lse_tol = 1e-4
     assert (lse.cpu()[fin] - want_lse[fin]).abs().max() <= lse_tol, tag + " LSE"
     check(qg.grad, qf.grad, dtype, tag + " dQ")
     check(kg.grad, kf.grad, dtype, tag + " dK")
@@ -146,14 +146,14 @@ def test_document_mask_long_row_equals_causal_attention_per_document(dev, D):
         g1 = ops.attention_backward(do[sl], q[sl], k[sl], v[sl], o1, lse1, mask_mode=ops.MASK_CAUSAL)
         tag = f"D{D} document [{a}, {b})"
         check(o[sl], o1, torch.bfloat16, tag + " O")
-        assert (lse[:, :, a:b] - lse1).abs().max() <= 4e-3, tag + " LSE (two kernel results, each within 2e-3)"
+        assert (lse[:, :, a:b] - lse1).abs().max() <= 2e-4, tag + " LSE (two kernel results, each within 1e-4)"
         for got, want, name in zip((dq, dk, dv), g1, ("dQ", "dK", "dV")):
             check(got[sl], want, torch.bfloat16, f"{tag} {name}")
         if b - a <= 4097:
             qc, kc, vc, dc = (t[sl].float().cpu() for t in (q, k, v, do))
             want_o, want_lse = oa.attention_with_lse(qc, kc, vc, oa.causal_mask(b - a, b - a, "cpu"))
             check(o[sl], want_o, torch.bfloat16, tag + " O against the oracle")
-            assert (lse[:, :, a:b].cpu() - want_lse).abs().max() <= 2e-3, tag + " LSE against the oracle"
+            assert (lse[:, :, a:b].cpu() - want_lse).abs().max() <= 1e-4, tag + " LSE against the oracle"
             wants = oa.attention_backward_explicit(dc, qc, kc, vc, want_o, want_lse, oa.causal_mask(b - a, b - a, "cpu"))
             for got, want, name in zip((dq, dk, dv), wants, ("dQ", "dK", "dV")):
                 check(got[sl], want, torch.bfloat16, f"{tag} {name} against the oracle")
@@ -437,7 +437,7 @@ def test_block_functions_compose_with_global_lse(dev, dtype):
     ops.attention_merge_(ro, rl, a.out, a.lse)
     ops.attention_merge_(ro, rl, b.out, b.lse)
     check(ro, full.out, dtype, "merged O")
-    assert (rl - full.lse).abs().max() <= (1e-5 if dtype == torch.float32 else 2e-3)
+    assert (rl - full.lse).abs().max() <= (1e-5 if dtype == torch.float32 else 1e-4)
     dq, dk, dv = flash_attn_dense_backward(do, q, k, v, full.out, full.lse, causal=False)
     dq1, dk1, dv1 = flash_attn_dense_backward(do, q, k[:, :, :64], v[:, :, :64], full.out, full.lse, causal=False)
     dq2, dk2, dv2 = flash_attn_dense_backward(do, q, k[:, :, 64:], v[:, :, 64:], full.out, full.lse, causal=False)

@@ -259,3 +259,24 @@ def test_optimizer_plumbing_on_host():
     assert model_param.grad is None
     mw.load_state_dict(sd)
     torch.testing.assert_close(model_param, torch.full_like(model_param, 3.0))
+
+
+def test_adjacent_gradient_columns_are_recognised():
+    """The one-product projections take their output gradients as one matrix when these already lie side by side."""
+    from maltos_amd.llama import _adjacent_columns
+
+    B, S, D = 2, 5, 4
+    joint = torch.arange(B * S * 8 * D, dtype=torch.float32).view(B, S, 8, D)
+    q, k, v = (joint[:, :, a:b].reshape(B, S, (b - a) * D) for a, b in ((0, 4), (4, 6), (6, 8)))
+    assert q.untyped_storage().data_ptr() == joint.untyped_storage().data_ptr()   # views, as autograd hands them over
+    both = _adjacent_columns([q, k, v])
+    assert both is not None and both.shape == (B * S, 8 * D) and torch.equal(both, joint.view(B * S, 8 * D))
+    assert both.untyped_storage().data_ptr() == joint.untyped_storage().data_ptr()
+    assert _adjacent_columns([k, v]) is None                    # rows wider than the two together
+    assert _adjacent_columns([q, v, k]) is None                 # another order than the columns
+    assert _adjacent_columns([q, k.clone(), v]) is None         # another buffer
+    assert _adjacent_columns([q.contiguous(), k.contiguous(), v.contiguous()]) is None
+    tail = torch.zeros(B, S, 8, D)[:, :, 4:]
+    assert _adjacent_columns([tail[:, :, :2].reshape(B, S, 2 * D), tail[:, :, 2:].reshape(B, S, 2 * D)]) is None
+    whole = torch.zeros(3, 6)
+    assert _adjacent_columns([whole[:, :2], whole[:, 2:]]).data_ptr() == whole.data_ptr()
