@@ -440,14 +440,18 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
     return out
 
 
-def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False):
+def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned_gemms=False):
     """graph=True: forward + backward replayed from one HIP graph (clip, AdamW and the gradient clear stay eager).
     zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
     per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer."""
+    from maltos_amd.gemm_tuning import tuned_gemms_off, use_tuned_gemms
     from maltos_amd.grad_clip import clip_grad_norm_fused_
     from maltos_amd.llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
     from maltos_amd.optim import FusedAdamW, MasterWeightsOptimizer
 
+    # the linear layers' products run on the vendor GEMM libraries; which of their kernels serves which shape comes from
+    # the selection the package ships for gfx950 (0: the file was recorded with other library versions and is not used)
+    gemm_shapes = 0 if no_tuned_gemms else use_tuned_gemms()
     cfg = LlamaConfig(vocab_size=32000, hidden_size=512, intermediate_size=1376, num_hidden_layers=8,
                       num_attention_heads=8, max_position_embeddings=2048, rms_norm_eps=1e-5)
     torch.manual_seed(1234)
@@ -498,12 +502,15 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False):
     # a fixed number of untimed steps (~0.3 s) in front: the three legs then report loss and gradient norm of the same
     # optimizer step, and they agree when the layouts compute the same thing
     sec = timed(torch, step_zero1 if zero1 else step_graph if graph else step, steps, warmup, preheat_steps=LLAMA_PREHEAT_STEPS)
+    tuned_gemms_off()
     tokens = 8 * 2048
     res = {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"].detach()),
            "grad_norm_last": float(out["norm"]) if zero1 else float(out["sq"].sqrt()),
            "optimizer_steps_taken": LLAMA_PREHEAT_STEPS + warmup + steps,
            "params": sum(p.numel() for p in model.parameters()),
-           "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12}
+           "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12,
+           "gemm_kernels": (f"per-shape selection of maltos_amd/tuned/gemm_gfx950.csv ({gemm_shapes} shapes)" if gemm_shapes
+                            else "the GEMM libraries' own choice")}
     if zero1:
         res["buckets"] = len(z.buckets)
     return res
@@ -696,6 +703,8 @@ def main() -> int:
         leg("hbm_kernels", lambda: bench_hbm_kernels(torch, ops, _lib, dev))
         leg("llama50m_train_step", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup)))
         leg("llama50m_train_step_graph", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), graph=True))
+        leg("llama50m_train_step_graph_library_gemm_choice",
+            lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), graph=True, no_tuned_gemms=True))
         leg("llama50m_train_step_zero1_layout", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), zero1=True))
         if not args.skip_cpu:
             leg("cfg1_tiny_llama_step_vs_cpu", lambda: cpu_baseline_llama(torch, dev, "cfg1"))

@@ -280,3 +280,17 @@ def test_adjacent_gradient_columns_are_recognised():
     assert _adjacent_columns([tail[:, :, :2].reshape(B, S, 2 * D), tail[:, :, 2:].reshape(B, S, 2 * D)]) is None
     whole = torch.zeros(3, 6)
     assert _adjacent_columns([whole[:, :2], whole[:, 2:]]).data_ptr() == whole.data_ptr()
+
+
+def test_shipped_gemm_selection_file_is_well_formed():
+    from maltos_amd.gemm_tuning import TUNED_FILE, use_tuned_gemms
+
+    rows = [line.split(",") for line in TUNED_FILE.read_text().splitlines()]
+    validators = {r[1] for r in rows if r[0] == "Validator"}
+    assert {"PT_VERSION", "HIP_VERSION", "HIPBLASLT_VERSION", "ROCBLAS_VERSION", "GCN_ARCH_NAME"} <= validators
+    assert any(r[0] == "Validator" and r[1] == "GCN_ARCH_NAME" and r[2].startswith("gfx950") for r in rows)
+    shapes = [r for r in rows if r[0].startswith("Gemm")]
+    assert len(shapes) >= 15 and all(len(r) == 4 and float(r[3]) > 0 for r in shapes)
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="needs a GPU"):
+            use_tuned_gemms()
