@@ -440,10 +440,13 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
     return out
 
 
-def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned_gemms=False):
+def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned_gemms=False, zero2=False):
     """graph=True: forward + backward replayed from one HIP graph (clip, AdamW and the gradient clear stay eager).
     zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
-    per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer."""
+    per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer.
+    zero2=True: ZeRO-2's per-bucket gradient buffers instead of one: every bucket's shard is taken when its last
+    gradient has arrived, inside the backward pass."""
+    zero1 = zero1 or zero2
     from maltos_amd.gemm_tuning import tuned_gemms_off, use_tuned_gemms
     from maltos_amd.grad_clip import clip_grad_norm_fused_
     from maltos_amd.llama import LlamaConfig, LlamaForCausalLM, set_grad_accumulation_into_buffers
@@ -466,7 +469,8 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned
         ps, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1))
     if zero1:
         from maltos_amd.zero1 import Zero1FlatBuffers
-        z = Zero1FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=25)
+        from maltos_amd.zero2 import Zero2FlatBuffers
+        z = (Zero2FlatBuffers if zero2 else Zero1FlatBuffers)(model, optimizer_factory=factory, bucket_mb_size=25)
     else:
         opt = factory(model.parameters())
     gen = torch.Generator().manual_seed(1234)
@@ -706,6 +710,7 @@ def main() -> int:
         leg("llama50m_train_step_graph_library_gemm_choice",
             lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), graph=True, no_tuned_gemms=True))
         leg("llama50m_train_step_zero1_layout", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), zero1=True))
+        leg("llama50m_train_step_zero2_layout", lambda: bench_llama50m(torch, dev, half, max(10, args.warmup), zero2=True))
         if not args.skip_cpu:
             leg("cfg1_tiny_llama_step_vs_cpu", lambda: cpu_baseline_llama(torch, dev, "cfg1"))
             leg("cfg5_llama50m_step_vs_cpu", lambda: cpu_baseline_llama(torch, dev, "cfg5"))

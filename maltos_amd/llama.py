@@ -102,7 +102,7 @@ class _SplitKLinearFn(torch.autograd.Function):
                 grad = None
             dw = _weight_grad(x.reshape(-1, x.shape[-1]), dy.reshape(-1, dy.shape[-1]), grad)
             if grad is not None:
-                notify_grad_written(weight)   # autograd's hooks on the weight do not fire for a gradient added here
+                notify_grad_written(weight)   # autograd's hooks on the weight see no gradient for what was added here
         return dx, dw, None
 
 
@@ -253,8 +253,9 @@ class HipLinear(nn.Linear):
 
     `accumulate_into_grad = True` (off by default; set it on the class or on an instance) makes the backward add dW
     straight into an existing `weight.grad` and return no gradient for the weight: one pass instead of two when the
-    gradients live in a flat buffer that is cleared, not dropped, between steps.  Autograd hooks on the weight do not
-    fire in that mode, so it is for callers that read the gradients from the buffer after backward."""
+    gradients live in a flat buffer that is cleared, not dropped, between steps.  Autograd hooks on the weight see no
+    gradient in that mode (they run with None), so it is for callers that read the gradients from the buffer after
+    backward; whoever needs to know that the buffer was written is told through `optim.notify_grad_written`."""
 
     accumulate_into_grad = False
 

@@ -18,7 +18,7 @@ world_size == 1 the reduce-scatter and the all-gather are the local copies the r
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable
 
 import torch
@@ -53,7 +53,7 @@ def role_params(model: nn.Module) -> list[nn.Parameter]:
     return [p for p in model.parameters() if p.requires_grad][::-1]
 
 
-@dataclass
+@dataclass(eq=False)   # a bucket is itself: comparing the tensors it holds field by field is never meant
 class Bucket:
     """zero1.py:24-36 without the process-group fields."""
 
@@ -64,6 +64,9 @@ class Bucket:
     shard_start: int
     shard_end: int
     local_param: nn.Parameter
+    # ZeRO-2 only (zero2.py:34-35 of the reference): reductions still to fire in this backward, per-micro-batch buffers
+    pending_exec_reductions: int = 0
+    exec_states: list = field(default_factory=list)
 
 
 ReduceScatter = Callable[[torch.Tensor, torch.Tensor], None]   # (out_shard, full_grad): out <- this rank's slice of the mean
@@ -78,6 +81,10 @@ class Zero1FlatBuffers:
     `runtime.create_optimizer` does in the reference (zero1.py:74-76); for bf16 models pass a factory that wraps them
     in `MasterWeightsOptimizer` (runtime/core.py:319-325).
     """
+
+    # ZeRO-1 keeps one gradient buffer laid out like the data buffer; a subclass that brings its own gradient buffers
+    # (ZeRO-2: one per bucket and micro-batch) turns this off and `grad_buffer` stays None
+    whole_model_grad_buffer = True
 
     def __init__(self, model: nn.Module, *, optimizer_factory: Callable[[list[nn.Parameter]], torch.optim.Optimizer],
                  world_size: int = 1, rank: int = 0, bucket_mb_size: int = 25,
@@ -108,7 +115,8 @@ class Zero1FlatBuffers:
         padded = [padded_len(sum(p.numel() for p in bucket), self.world_size) for bucket in param_buckets]
         total = sum(padded)
         self.data_buffer = torch.zeros(total, dtype=dtype, device=device)
-        self.grad_buffer = torch.zeros(total, dtype=dtype, device=device)
+        if self.whole_model_grad_buffer:
+            self.grad_buffer = torch.zeros(total, dtype=dtype, device=device)
         offset = 0
         for bucket_params, padded_size in zip(param_buckets, padded):
             cursor = offset
@@ -117,7 +125,8 @@ class Zero1FlatBuffers:
                 with torch.no_grad():
                     self.data_buffer[cursor:cursor + n].copy_(param.detach().reshape(-1))
                     param.data = self.data_buffer[cursor:cursor + n].view_as(param)
-                    param.grad = self.grad_buffer[cursor:cursor + n].view_as(param)
+                    if self.grad_buffer is not None:
+                        param.grad = self.grad_buffer[cursor:cursor + n].view_as(param)
                 cursor += n
             per_rank = padded_size // self.world_size
             shard_start = offset + self.rank * per_rank
@@ -205,8 +214,9 @@ class Zero1FlatBuffers:
     # ---- POST_STEP: zero1.py:236-260 --------------------------------------------------------------------------
     def gather_updated_params(self) -> None:
         """Updated shards back into the flat data buffer (the model's parameters are views of it); grads zeroed."""
-        assert self.data_buffer is not None and self.grad_buffer is not None
-        self.grad_buffer.zero_()
+        assert self.data_buffer is not None
+        if self.grad_buffer is not None:
+            self.grad_buffer.zero_()
         with torch.no_grad():
             for bucket in self.buckets:
                 local = bucket.local_param.detach().contiguous()

@@ -90,6 +90,39 @@ def test_flat_and_zero1_layouts_take_the_same_step(dev, accumulate):
         assert lf == lz and abs(nf - nz) <= 1e-12 * nf
 
 
+@pytest.mark.parametrize("accumulate", [False, True], ids=["autograd-accumulation", "accumulate-into-buffers"])
+def test_zero2_bucket_buffers_take_the_zero1_step(dev, accumulate):
+    """ZeRO-2 keeps the gradients in per-bucket buffers and takes every bucket's shard in when its last gradient has
+    arrived; on one rank that is the ZeRO-1 step bit for bit.  From the second step on the parameters' gradients are
+    bound, and with accumulate_into_grad the linear layers then add straight into the bucket buffers, past autograd's
+    hooks: the buckets still complete (through the gradient-written notification)."""
+    from maltos_amd.zero2 import Zero2FlatBuffers
+
+    one = _model(dev, layers=2)
+    two = copy.deepcopy(one)
+    if accumulate:
+        set_grad_accumulation_into_buffers(one)
+        set_grad_accumulation_into_buffers(two)
+    z1 = Zero1FlatBuffers(one, optimizer_factory=_factory, bucket_mb_size=25)
+    z2 = Zero2FlatBuffers(two, optimizer_factory=_factory, bucket_mb_size=25)
+    assert z2.grad_buffer is None and len(z2.buckets) == len(z1.buckets)
+    for step in range(3):
+        batch = _batch(dev, seed=77 + step, rows=2, seq=512)
+        z1.reset_grads()
+        loss1 = one(batch)
+        loss1.backward()
+        z2.reset_grads()
+        loss2 = two(batch)
+        loss2.backward()
+        assert sorted(z2.fired_order) == list(range(len(z2.buckets))), f"step {step}: every bucket completes inside the backward pass"
+        assert loss1.item() == loss2.item()
+        norm1, norm2 = z1.step(1.0), z2.step(1.0)
+        assert norm1 == norm2
+        assert torch.equal(z1.data_buffer, z2.data_buffer), f"step {step}"
+        for b1, b2 in zip(z1.buckets, z2.buckets):
+            assert torch.equal(b1.local_param.detach(), b2.local_param.detach())
+
+
 def test_device_side_clip_takes_the_same_steps_as_host_side_clip(dev):
     """clip_grad_norm_fused_ (norm stays on the device, the AdamW kernel applies the coefficient) against clip_grad_norm_
     (host reads the norm, a scaling pass, then the step): bit-equal masters over steps that do and do not clip."""
