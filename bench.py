@@ -618,8 +618,11 @@ def cpu_baseline_llama(torch, dev, which):
         opt.step()
         opt.zero_grad(set_to_none=True)
 
+    from maltos_amd.gemm_tuning import tuned_gemms_off, use_tuned_gemms
+    gemm_shapes = use_tuned_gemms() if which == "cfg5" else 0   # as the llama50m_train_step leg; the parity step below too
     step(timed_step=False)
     gpu_sec = timed(torch, step, 10, 3, preheat_steps=LLAMA_PREHEAT_STEPS)
+    tuned_gemms_off()
     tokens = batch * seq
     return {"workload": f"{'tiny LLaMA fp32 (configuration 1)' if which == 'cfg1' else 'LLaMA-50M bf16 (configuration 5)'} full train step, "
                         f"batch {batch} x {seq}",
@@ -627,6 +630,8 @@ def cpu_baseline_llama(torch, dev, which):
                     "sample": f"oracle.llama.train_step (fp32 PyTorch restatement, stock AdamW) at full size, {timed_steps} timed step(s)"
                               + (", 1 warm-up" if which == "cfg1" else ", no warm-up")},
             "gpu": {"ms": gpu_sec * 1e3, "tokens_per_sec": tokens / gpu_sec,
+                    "gemm_kernels": (f"per-shape selection of maltos_amd/tuned/gemm_gfx950.csv ({gemm_shapes} shapes)" if gemm_shapes
+                                     else "the GEMM libraries' own choice"),
                     "clip": "none (the configuration has no clip)" if max_norm is None else
                             "global-norm clip at 1.0 applied on the device (no host read): the eager step of extra.llama50m_train_step"},
             "parity": {"loss": {"hip": first["loss"], "oracle": want_loss, "rel": abs(first["loss"] - want_loss) / abs(want_loss)},
