@@ -99,7 +99,16 @@ def run(args: argparse.Namespace) -> dict:
     set_grad_accumulation_into_buffers(model)   # weight gradients add into bound gradient buffers where there are any
     adamw = lambda ps: FusedAdamW(ps, lr=args.lr, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
     factory = (lambda ps: MasterWeightsOptimizer(ps, optimizer_factory=adamw)) if dtype == torch.bfloat16 else adamw
-    zero = Zero1FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=args.bucket_mb) if args.optimizer_layout == "zero1" else None
+    zero = None
+    if args.optimizer_layout == "zero1":
+        zero = Zero1FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=args.bucket_mb)
+    elif args.optimizer_layout == "zero2":
+        from .zero2 import Zero2FlatBuffers
+        zero = Zero2FlatBuffers(model, optimizer_factory=factory, bucket_mb_size=args.bucket_mb)
+    gemm_shapes = 0
+    if not args.library_gemm_choice:
+        from .gemm_tuning import use_tuned_gemms
+        gemm_shapes = use_tuned_gemms()   # 0: the shipped selection does not fit this GEMM library version and is not used
     opt = None if zero else factory(list(model.parameters()))
 
     if args.shards:
@@ -154,6 +163,7 @@ def run(args: argparse.Namespace) -> dict:
     return {
         "model": args.model, "dtype": args.dtype, "batch_size": args.batch_size, "seq_len": args.seq_len, "data": source,
         "optimizer_layout": args.optimizer_layout, "graph": bool(args.graph), "buckets": len(zero.buckets) if zero else None,
+        "gemm_shapes_selected_from_file": gemm_shapes,
         "params": sum(p.numel() for p in model.parameters()), "steps": args.steps, "warmup": args.warmup,
         "step_ms_mean": mean * 1e3, "step_ms_median": statistics.median(times) * 1e3, "step_ms_min": min(times) * 1e3,
         "tokens_per_sec": tokens / mean, "model_tflops": tokens * model.flops_per_token() / mean / 1e12,
@@ -166,7 +176,10 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     ap.add_argument("--model", choices=sorted(MODELS), default="llama-50m")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--layout", choices=["dense", "packed"], default="dense")
-    ap.add_argument("--optimizer-layout", choices=["flat", "zero1"], default="flat")
+    ap.add_argument("--optimizer-layout", choices=["flat", "zero1", "zero2"], default="flat")
+    ap.add_argument("--library-gemm-choice", action="store_true",
+                    help="leave the choice of GEMM kernels to hipBLASLt / rocBLAS instead of the per-shape selection "
+                         "shipped for gfx950 (maltos_amd.gemm_tuning)")
     ap.add_argument("--graph", action="store_true",
                     help="replay forward + backward from one HIP graph (bf16, fixed batch shapes; see maltos_amd.graph_step)")
     ap.add_argument("--bucket-mb", type=int, default=25)
