@@ -437,6 +437,25 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
             us = total_ms / max(1, launches) * 1e3
             gbps = nbytes / (us * 1e-6) / 1e9
             out[label] = {"us": us, "algorithmic_bytes": nbytes, "gbps": gbps, "frac_of_hbm_peak": gbps / HBM_PEAK_GBPS}
+        # yardstick: what a plain device-to-device copy (torch's copy kernel) reaches when it moves as many bytes as the
+        # small kernels above, timed the same way (an event pair around every launch): launches this short are bounded by
+        # how fast a grid starts and drains, whatever they compute
+        for label, n_elem in (("plain_copy_moving_33.6MB", N * h), ("plain_copy_moving_67.1MB", 2 * N * h)):
+            src = torch.randn(n_elem, generator=g).to(bf).to(dev)
+            dst = torch.empty_like(src)
+            fn = lambda: dst.copy_(src)
+            preheat(torch, fn, 0.05)
+            pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            torch.cuda.synchronize()
+            for a, b in pairs:
+                a.record()
+                fn()
+                b.record()
+            torch.cuda.synchronize()
+            us = sum(a.elapsed_time(b) for a, b in pairs) / reps * 1e3
+            nbytes = 2 * n_elem * e
+            out[label] = {"us": us, "algorithmic_bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9,
+                          "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS}
     return out
 
 
