@@ -172,6 +172,22 @@ def test_document_mask_drawn_shapes(dev, seed):
              pad_tail=draw(0, min(40, S - 1)), share_ids=bool(seed % 3))
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_causal_and_unmasked_drawn_shapes(dev, seed):
+    """Drawn batch sizes, head groupings, head dims (the MFMA kernels' 64 and 128 and the generic kernels' others), query
+    and key lengths that differ either way (bottom-right aligned causal mask: with more queries than keys the first rows
+    see nothing and must come out as zeros with LSE = -inf), both dtypes."""
+    gen = torch.Generator().manual_seed(3000 + seed)
+    draw = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    B, Hkv, group = draw(1, 3), draw(1, 2), (1, 2, 4, 8)[draw(0, 3)]
+    D = (64, 128, 64, 128, 32, 96, 192, 16)[seed % 8]
+    dtype = torch.float32 if seed % 8 == 7 else torch.bfloat16
+    Sq = (draw(1, 70), draw(71, 400), draw(401, 1100))[draw(0, 2)]
+    Sk = (Sq, draw(1, 1100), Sq + draw(1, 200))[draw(0, 2)]
+    mode = ops.MASK_CAUSAL if seed % 2 == 0 else ops.MASK_NONE
+    run_case(dev, dtype, B, Hkv * group, Hkv, Sq, Sk, D, mode, 4000 + seed)
+
+
 @pytest.mark.parametrize("D", [64, 128])
 def test_document_plan_is_reused_and_follows_the_ids(dev, D):
     """The plan built for a call's ids (mlts_attn_doc_plan) serves later calls with the same id tensors, gives the results
