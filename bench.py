@@ -462,7 +462,8 @@ def bench_hbm_kernels(torch, ops, _lib, dev, reps=20):
 def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned_gemms=False, zero2=False):
     """graph=True: forward + backward replayed from one HIP graph (clip, AdamW and the gradient clear stay eager).
     zero1=True: the same step with the parameters in the ZeRO-1 flat buffers (world size 1): one optimizer launch
-    per 25 MiB bucket on the bucket's local shard, host read of the norm, gather back into the flat data buffer.
+    per 25 MiB bucket on the bucket's local shard, the clip applied on the device as in the flat legs, gather back into
+    the flat data buffer.
     zero2=True: ZeRO-2's per-bucket gradient buffers instead of one: every bucket's shard is taken when its last
     gradient has arrived, inside the backward pass."""
     zero1 = zero1 or zero2
@@ -519,7 +520,7 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned
         z.reset_grads()
         loss = model(batch)
         loss.backward()
-        out["norm"] = z.step(1.0)
+        out["norm"] = z.step(1.0, clip_on_device=True)   # the sum of squares, left on the device as in the flat legs
         out["loss"] = loss
 
     # a fixed number of untimed steps (~0.3 s) in front: the three legs then report loss and gradient norm of the same
@@ -528,7 +529,7 @@ def bench_llama50m(torch, dev, steps, warmup, zero1=False, graph=False, no_tuned
     tuned_gemms_off()
     tokens = 8 * 2048
     res = {"ms_per_step": sec * 1e3, "tokens_per_sec": tokens / sec, "loss_last": float(out["loss"].detach()),
-           "grad_norm_last": float(out["norm"]) if zero1 else float(out["sq"].sqrt()),
+           "grad_norm_last": float(out["norm"].sqrt()) if zero1 else float(out["sq"].sqrt()),
            "optimizer_steps_taken": LLAMA_PREHEAT_STEPS + warmup + steps,
            "params": sum(p.numel() for p in model.parameters()),
            "tflops_reference_estimator": tokens * model.flops_per_token() / sec / 1e12,

@@ -211,6 +211,24 @@ class Zero1FlatBuffers:
         self.grad_norm = global_norm
         return global_norm
 
+    def clip_local_shards_on_device(self, max_norm: float) -> torch.Tensor:
+        """The same clip without the host reading the norm: the fp64 sum of squares of all shards stays on the device
+        (summed over the ranks by `all_reduce_sum`) and the fused AdamW kernel applies max_norm / (norm + 1e-6) to the
+        gradients it reads when that is below 1.  Returns the device scalar (its square root is the norm).  Needs the
+        fp32 master copy of `MasterWeightsOptimizer` over `FusedAdamW`; a non-finite norm is not detected here."""
+        from .grad_clip import global_grad_sq_norm
+        inner = getattr(self.optimizer, "_optimizer", self.optimizer)
+        set_clip = getattr(inner, "set_clip", None)
+        if not callable(set_clip) or getattr(self.optimizer, "flat_master_grad", None) is None:
+            raise TypeError("clip_local_shards_on_device needs MasterWeightsOptimizer over FusedAdamW as the shards' optimizer")
+        sq = global_grad_sq_norm(self.optimizer)
+        if sq is None:
+            raise ValueError("no gradients to clip")
+        if self.world_size > 1:
+            self._all_reduce_sum(sq)
+        set_clip(sq, float(max_norm))
+        return sq
+
     # ---- POST_STEP: zero1.py:236-260 --------------------------------------------------------------------------
     def gather_updated_params(self) -> None:
         """Updated shards back into the flat data buffer (the model's parameters are views of it); grads zeroed."""
@@ -236,9 +254,11 @@ class Zero1FlatBuffers:
             resync()
 
     # ---- the phases of one optimizer step in the reference's order --------------------------------------------
-    def step(self, max_norm: float | None = None) -> float | None:
+    def step(self, max_norm: float | None = None, *, clip_on_device: bool = False) -> "float | torch.Tensor | None":
+        """Returns the gradient norm as the reference's metadata has it (a host float), or with `clip_on_device` the
+        device scalar sum of squares, which nobody has to wait for."""
         self.reduce_grads()
-        norm = self.clip_local_shards(max_norm)
+        norm = self.clip_local_shards_on_device(max_norm) if clip_on_device and max_norm is not None else self.clip_local_shards(max_norm)
         assert self.optimizer is not None
         self.optimizer.step()
         self.gather_updated_params()

@@ -123,6 +123,28 @@ def test_zero2_bucket_buffers_take_the_zero1_step(dev, accumulate):
             assert torch.equal(b1.local_param.detach(), b2.local_param.detach())
 
 
+def test_zero_layout_clip_on_device_takes_the_host_clip_steps(dev):
+    """`step(max_norm, clip_on_device=True)` (norm left on the device, coefficient applied by the AdamW kernel) against the
+    reference's order (host reads the norm, scales the shards, steps): bit-equal parameters over steps that do and do not clip."""
+    a = _model(dev, layers=2)
+    b = copy.deepcopy(a)
+    za = Zero1FlatBuffers(a, optimizer_factory=_factory, bucket_mb_size=25)
+    zb = Zero1FlatBuffers(b, optimizer_factory=_factory, bucket_mb_size=25)
+    clipped = 0
+    for step in range(6):
+        batch = _batch(dev, seed=5, rows=2, seq=512)
+        for z, m in ((za, a), (zb, b)):
+            z.reset_grads()
+            m(batch).backward()
+        max_norm = 1.0 if step % 2 == 0 else 100.0
+        norm = za.step(max_norm)
+        sq = zb.step(max_norm, clip_on_device=True)
+        clipped += norm > max_norm
+        assert abs(float(sq.sqrt()) - norm) <= 1e-12 * norm
+        assert torch.equal(za.data_buffer, zb.data_buffer), f"step {step} (norm {norm:.3f})"
+    assert 1 <= clipped < 6
+
+
 def test_device_side_clip_takes_the_same_steps_as_host_side_clip(dev):
     """clip_grad_norm_fused_ (norm stays on the device, the AdamW kernel applies the coefficient) against clip_grad_norm_
     (host reads the norm, a scaling pass, then the step): bit-equal masters over steps that do and do not clip."""
