@@ -365,3 +365,59 @@ def test_model_keeps_hooked_logits(dev):
         results[form] = (loss.detach().clone(), model.lm_head.weight.grad.clone())
     for form in ("hooked", "config-off"):
         assert torch.equal(results[form][0], results["own"][0]) and torch.equal(results[form][1], results["own"][1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_empty_inputs_are_served(dev, dtype):
+    """Zero rows, zero batch, zero length: every op returns outputs of the right shape (and gradients of the right shape
+    through its backward) without launching into nothing; a loss over no rows is 0."""
+    h, I, V, H, D = 256, 384, 512, 2, 64
+    w = torch.ones(h, dtype=dtype, device=dev, requires_grad=True)
+    x = torch.zeros(0, h, dtype=dtype, device=dev, requires_grad=True)
+    y = ops.rms_norm(x, w, 1e-5)
+    y.sum().backward()
+    assert y.shape == (0, h) and x.grad.shape == (0, h) and w.grad.shape == (h,) and w.grad.abs().max() == 0
+    s, y2 = ops.add_rms_norm(x, x, w, 1e-5)
+    assert s.shape == (0, h) and y2.shape == (0, h)
+    (s.sum() + y2.sum()).backward()
+
+    cos = torch.ones(16, D // 2, dtype=dtype, device=dev)
+    sin = torch.zeros(16, D // 2, dtype=dtype, device=dev)
+    for shape in ((0, H, 8, D), (2, H, 0, D)):
+        q = torch.zeros(shape, dtype=dtype, device=dev, requires_grad=True)
+        k = torch.zeros(shape, dtype=dtype, device=dev, requires_grad=True)
+        r = ops.rope(q, cos, sin)
+        rq, rk = ops.rope_pair(q, k, cos, sin)
+        (r.sum() + rq.sum() + rk.sum()).backward()
+        assert r.shape == shape and rq.shape == shape and q.grad.shape == shape
+        for mode in (ops.MASK_CAUSAL, ops.MASK_NONE):
+            o, lse = ops.attention(q, k, k, mask_mode=mode, return_lse=True)
+            o.sum().backward()
+            assert o.shape == shape and lse.shape == shape[:3] and k.grad.shape == shape
+
+    # queries without any key: zeros and LSE = -inf; keys without any query: zero gradients
+    q = torch.randn(1, H, 5, D, device=dev).to(dtype).requires_grad_(True)
+    k0 = torch.zeros(1, H, 0, D, dtype=dtype, device=dev, requires_grad=True)
+    o, lse = ops.attention(q, k0, k0, mask_mode=ops.MASK_NONE, return_lse=True)
+    o.sum().backward()
+    assert o.abs().max() == 0 and torch.isinf(lse).all() and (lse < 0).all() and q.grad.abs().max() == 0 and k0.grad.shape == k0.shape
+
+    g = torch.zeros(0, I, dtype=dtype, device=dev, requires_grad=True)
+    u = torch.zeros(0, I, dtype=dtype, device=dev, requires_grad=True)
+    hh = ops.swiglu(g, u)
+    hh.sum().backward()
+    assert hh.shape == (0, I) and g.grad.shape == (0, I)
+
+    logits = torch.zeros(0, V, dtype=dtype, device=dev, requires_grad=True)
+    loss = ops.cross_entropy(logits, torch.zeros(0, dtype=torch.long, device=dev))
+    loss.backward()
+    assert float(loss.detach()) == 0.0 and logits.grad.shape == (0, V)
+
+    if dtype == torch.float32:
+        p = torch.zeros(0, device=dev)
+        ops.adamw_step_(p, p.clone(), p.clone(), p.clone(), lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=1)
+        assert float(ops.sq_norm(p)) == 0.0
+        ops.scale_(p, 0.5)
+        ops.grad_to_f32_(p, torch.zeros(0, dtype=torch.bfloat16, device=dev))
+    out_acc = torch.zeros(1, H, 0, D, device=dev)
+    ops.attention_merge_(out_acc, torch.zeros(1, H, 0, device=dev), torch.zeros(1, H, 0, D, dtype=dtype, device=dev), torch.zeros(1, H, 0, device=dev))
