@@ -742,3 +742,28 @@ def test_all_gather_kv_core_matches_global_attention(dev, packed):
             dv_sum.index_add_(2, idx[src], v.grad.float().cpu())
     assert ((dk_sum - gk.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gk.grad.abs())).all()
     assert ((dv_sum - gv.grad).abs() <= 4 * (2e-2 + 2.0 ** -8 * gv.grad.abs())).all()
+
+
+def test_tensors_of_more_than_two_to_the_31_elements(dev):
+    """q, k, v of 2^31 elements each (B=4, H=32, S=131072, D=128: element offsets past 32 bits): the first and the last
+    (batch, head) pair come out exactly as from a call on that pair alone, forward and backward; a size-independent
+    property where the oracle cannot go."""
+    B, H, S, D = 4, 32, 131072, 128
+    gen = torch.Generator(device=dev).manual_seed(11)
+    q, k, v, do = (torch.randn(B, S, H, D, generator=gen, device=dev, dtype=torch.bfloat16).transpose(1, 2) for _ in range(4))
+    assert q.numel() == 2 ** 31
+    o, lse = ops.attention_forward(q, k, v, mask_mode=ops.MASK_CAUSAL)
+    dq, dk, dv = ops.attention_backward(do, q, k, v, o, lse, mask_mode=ops.MASK_CAUSAL)
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        o1, lse1 = ops.attention_forward(q[sl], k[sl], v[sl], mask_mode=ops.MASK_CAUSAL)
+        assert torch.equal(o[sl], o1) and torch.equal(lse[sl], lse1), (b, h)
+        for got, want, name in zip((dq, dk, dv), ops.attention_backward(do[sl], q[sl], k[sl], v[sl], o1, lse1, mask_mode=ops.MASK_CAUSAL),
+                                   ("dQ", "dK", "dV")):
+            assert torch.equal(got[sl], want), (b, h, name)
+    # and the last rows against the oracle: the last 64 queries of the last pair see all 131072 keys
+    sl = (slice(B - 1, B), slice(H - 1, H))
+    qf, kf, vf = q[sl][:, :, -64:].float().cpu(), k[sl].float().cpu(), v[sl].float().cpu()
+    want_o, want_lse = oa.attention_with_lse(qf, kf, vf, oa.causal_mask(64, S, "cpu"))
+    check(o[sl][:, :, -64:], want_o, torch.bfloat16, "last rows O")
+    assert (lse[sl][:, :, -64:].cpu() - want_lse).abs().max() <= 1e-4

@@ -421,3 +421,74 @@ def test_empty_inputs_are_served(dev, dtype):
         ops.grad_to_f32_(p, torch.zeros(0, dtype=torch.bfloat16, device=dev))
     out_acc = torch.zeros(1, H, 0, D, device=dev)
     ops.attention_merge_(out_acc, torch.zeros(1, H, 0, device=dev), torch.zeros(1, H, 0, D, dtype=dtype, device=dev), torch.zeros(1, H, 0, device=dev))
+
+
+def test_more_than_two_to_the_31_elements(dev):
+    """Tensors of more than 2^31 elements (flat indices past 32 bits): the head, the middle that straddles the 2^31st
+    element and the tail of every result equal what the same kernel gives for those rows alone."""
+    torch.manual_seed(5)
+    # cross-entropy: 70,000 x 32,000 = 2.24e9 logits
+    rows, V = 70_000, 32_000
+    logits = torch.randn(rows, V, device=dev, dtype=torch.bfloat16)
+    labels = torch.randint(0, V, (rows,), device=dev)
+    labels[::7] = -100
+    loss, dlogits, count = torch.ops.maltos.ce_fwd_bwd(logits, labels, -100)   # mean over the rows that have a target
+    parts = 0.0
+    cut = (2 ** 31) // V
+    for a, b in ((0, 300), (cut - 150, cut + 150), (rows - 300, rows)):
+        s, d, c = torch.ops.maltos.ce_fwd_bwd(logits[a:b].contiguous(), labels[a:b].contiguous(), -100)
+        # the gradient carries 1 / count of its own call
+        assert torch.allclose(dlogits[a:b].float() * float(count), d.float() * float(c), rtol=2 ** -7, atol=1e-6), (a, b)
+    for a in range(0, rows, 10_000):
+        s, _, c = torch.ops.maltos.ce_fwd_bwd(logits[a:a + 10_000].contiguous(), labels[a:a + 10_000].contiguous(), -100)
+        parts += float(s) * float(c)
+    assert int(count) == int((labels != -100).sum()) and abs(float(loss) * float(count) - parts) <= 1e-5 * parts
+    del logits, dlogits
+
+    # SwiGLU and RMSNorm: 4,400,000 rows of 512
+    n_rows, h = 4_400_000, 512
+    cut = (2 ** 31) // h
+    g = torch.randn(n_rows, h, device=dev, dtype=torch.bfloat16)
+    u = torch.randn(n_rows, h, device=dev, dtype=torch.bfloat16)
+    w = torch.randn(h, device=dev, dtype=torch.bfloat16)
+    out = torch.ops.maltos.swiglu_fwd(g, u)
+    y, rstd = torch.ops.maltos.rmsnorm_fwd(g, w, 1e-5)
+    dg, du = torch.ops.maltos.swiglu_bwd(out, g, u)
+    dx, dw = torch.ops.maltos.rmsnorm_bwd(u, g, w, rstd)
+    for a, b in ((0, 200), (cut - 100, cut + 100), (n_rows - 200, n_rows)):
+        ga, ua = g[a:b].contiguous(), u[a:b].contiguous()
+        assert torch.equal(out[a:b], torch.ops.maltos.swiglu_fwd(ga, ua))
+        ya, ra = torch.ops.maltos.rmsnorm_fwd(ga, w, 1e-5)
+        assert torch.equal(y[a:b], ya) and torch.equal(rstd[a:b], ra)
+        dga, dua = torch.ops.maltos.swiglu_bwd(out[a:b].contiguous(), ga, ua)
+        assert torch.equal(dg[a:b], dga) and torch.equal(du[a:b], dua)
+        assert torch.equal(dx[a:b], torch.ops.maltos.rmsnorm_bwd(ua, ga, w, ra)[0])
+    assert torch.isfinite(dw.float()).all()
+    del g, u, out, y, dg, du, dx
+
+    # AdamW, the norm and the gradient conversion over 2.2e9 parameters
+    n = 2 ** 31 + 4096 * 13 + 5
+    p = torch.randn(n, device=dev)
+    grad16 = torch.randn(n, device=dev, dtype=torch.bfloat16)
+    grad = torch.empty(n, device=dev)
+    sq = torch.zeros((), dtype=torch.float64, device=dev)
+    ops.grad_to_f32_(grad, grad16, sq_out=sq)
+    want_sq = sum(float(grad16[a:a + 2 ** 28].double().pow(2).sum()) for a in range(0, n, 2 ** 28))
+    assert abs(float(sq) - want_sq) <= 1e-9 * want_sq and abs(float(ops.sq_norm(grad)) - want_sq) <= 1e-9 * want_sq
+    m, v = torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+    hp = dict(lr=1e-2, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=1)
+    for a, b in ((0, 4096), (2 ** 31 - 2048, 2 ** 31 + 2048), (n - 4101, n)):
+        a -= a % 4   # 16-byte aligned views, like the whole buffer
+        pa, ga = p[a:b].clone(), grad[a:b].clone()
+        ma, va = torch.zeros_like(pa), torch.zeros_like(pa)
+        ops.adamw_step_(pa, ga, ma, va, **hp)
+        if a == 0:
+            first = (pa, ma, va)
+        elif b == n:
+            last = (a, pa, ma, va)
+        else:
+            mid = (a, b, pa, ma, va)
+    ops.adamw_step_(p, grad, m, v, **hp)
+    assert all(torch.equal(x[:4096], y) for x, y in zip((p, m, v), first))
+    assert all(torch.equal(x[mid[0]:mid[1]], y) for x, y in zip((p, m, v), mid[2:]))
+    assert all(torch.equal(x[last[0]:], y) for x, y in zip((p, m, v), last[1:]))
